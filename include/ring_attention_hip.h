@@ -1,0 +1,163 @@
+/*
+ * ring_attention_hip.h - C ABI of the MI355X (gfx950) ring-attention block-step library.
+ *
+ * The library replaces the per-device block step that the reference's ring_attention runs
+ * at every ring rotation, plus the carry initialisation / finalisation around it.  Every
+ * entry point below names the reference interface it stands in for (paths are relative to
+ * the reference checkout, package ring_attention/).  The reference has no C/FFI layer of
+ * its own: its plug point is the pair of Python callables selected by `block_impl`
+ * (ring.py:296-312), so these are the functions an FFI binding for that plug point binds.
+ *
+ * Conventions
+ *  - plain C types only; all pointers are DEVICE pointers unless stated otherwise;
+ *  - the caller owns every buffer; no entry point allocates or frees device memory;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream); work is
+ *    enqueued asynchronously on it and the call returns without synchronising;
+ *  - return value: RA_OK (0) or a negative RA_ERR_* code; argument validation happens
+ *    before any HIP call, so invalid arguments are rejected without touching a GPU;
+ *    ra_last_error() returns a thread-local description of the last failure;
+ *  - q/k/v/do/out tensors are bf16 with the head dimension contiguous; the batch, head and
+ *    length strides are given in ELEMENTS, so both the public [b, l, h, d] layout
+ *    (ring.py:80-82) and the internal [b, h, l, d] layout (ring.py:96-98) are accepted
+ *    without a transpose;
+ *  - carries and accumulators are fp32 and contiguous: o/dq/dk/dv [B, H, L, D],
+ *    m/l/lse/delta [B, H, L];
+ *  - D must be 64 or 128 and equal for q, k and v (the reference's kernels assume
+ *    dk == dv too, ring_kernel.py:170,175); lengths may be any positive number.
+ */
+#ifndef RING_ATTENTION_HIP_H
+#define RING_ATTENTION_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RA_OK 0
+#define RA_ERR_NULL (-1)        /* a required pointer is NULL                       */
+#define RA_ERR_SHAPE (-2)       /* a dimension is not positive / too large          */
+#define RA_ERR_HEAD_DIM (-3)    /* D is not 64 or 128                               */
+#define RA_ERR_ALIGN (-4)       /* pointer or stride breaks the 16-byte row rule    */
+#define RA_ERR_BIAS (-5)        /* inconsistent bias description                    */
+#define RA_ERR_HIP (-6)         /* a HIP runtime call failed (see ra_last_error)    */
+#define RA_ERR_DTYPE (-7)       /* unknown output dtype code                        */
+
+/* Bias terms, OR-ed into ra_bias.flags.  They are the device-side form of the reference's
+ * bias_fn (ring.py:107,186): each term is evaluated per score tile from token positions
+ * and per-token ids instead of being materialised as a dense [b, h, lq, lk] block. */
+#define RA_BIAS_CAUSAL 1   /* kv_pos <= q_pos                  (ring.py:393-397)            */
+#define RA_BIAS_WINDOW 2   /* |q_pos - kv_pos| < window (one-sided when CAUSAL is set)    */
+#define RA_BIAS_SEGMENT 4  /* q_segment_id == kv_segment_id    (ring.py:388-391)            */
+#define RA_BIAS_PREFIX 8   /* (q_prefix & kv_prefix) | kv_pos <= q_pos (ring.py:399-406)    */
+#define RA_BIAS_ALIBI 16   /* additive -slope[h] * |q_pos - kv_pos|                       */
+
+#define RA_DTYPE_BF16 0
+#define RA_DTYPE_F32 1
+
+/* bf16 tensor view [B, H, L, D] with explicit element strides (D contiguous). */
+typedef struct ra_tensor {
+  const void* ptr;
+  int64_t stride_b;
+  int64_t stride_h;
+  int64_t stride_l;
+} ra_tensor;
+
+/* Bias description for one (query shard, key/value shard) pair.
+ * Positions are implicit: token i of the query shard has position q_offset + i, token j
+ * of the key/value shard has position kv_offset + j (the shard's place in the ring).
+ * Per-token arrays are int32 [B, L] with a batch stride in elements; the kv-side arrays
+ * travel with the key/value shard, the q-side arrays with the query shard, exactly as
+ * bias_kv_kwargs / bias_q_kwargs rotate in the reference (ring.py:120,195). */
+typedef struct ra_bias {
+  int32_t flags;
+  int32_t window;
+  int64_t q_offset;
+  int64_t kv_offset;
+  const int32_t* q_segment_ids;
+  const int32_t* kv_segment_ids;
+  int64_t q_segment_stride_b;
+  int64_t kv_segment_stride_b;
+  const int32_t* q_prefix;
+  const int32_t* kv_prefix;
+  int64_t q_prefix_stride_b;
+  int64_t kv_prefix_stride_b;
+  const float* alibi_slopes; /* [H] */
+} ra_bias;
+
+/* One ring step of the forward pass. */
+typedef struct ra_fwd_step_params {
+  int32_t B, H, Lq, Lk, D;
+  float sm_scale;
+  ra_tensor q, k, v;
+  float* o; /* [B,H,Lq,D] unnormalised output carry, updated in place */
+  float* m; /* [B,H,Lq]   running row maximum of the biased, scaled scores */
+  float* l; /* [B,H,Lq]   running row sum of exp(score - m) */
+  ra_bias bias;
+} ra_fwd_step_params;
+
+/* One ring step of the backward pass. */
+typedef struct ra_bwd_step_params {
+  int32_t B, H, Lq, Lk, D;
+  float sm_scale;
+  ra_tensor q, k, v, dout;
+  const float* lse;   /* [B,H,Lq] m + log(l) of the whole forward pass */
+  const float* delta; /* [B,H,Lq] from ra_bwd_delta */
+  float* dq;          /* [B,H,Lq,D] accumulated in place (owned by the query shard)    */
+  float* dk;          /* [B,H,Lk,D] accumulated in place (owned by the key/value shard) */
+  float* dv;          /* [B,H,Lk,D] accumulated in place */
+  ra_bias bias;
+} ra_bwd_step_params;
+
+/* Version of this ABI (major * 1000 + minor). */
+int ra_version(void);
+/* Thread-local text for the last error returned on this thread ("" if none). */
+const char* ra_last_error(void);
+
+/* Carry initialisation o = 0, l = 0, m = -inf.          Replaces ring.py:124-126. */
+int ra_fwd_init(float* o, float* m, float* l, int32_t B, int32_t H, int32_t Lq, int32_t D,
+                void* stream);
+
+/* (o, m, l) <- online-softmax update with one key/value shard.
+ * Replaces fwd_block (ring_kernel.py:123-199) / _fwd_block (ring.py:58-76) together with
+ * the bias_fn call in front of it (ring.py:107).  Fully masked score tiles are skipped. */
+int ra_fwd_step(const ra_fwd_step_params* p, void* stream);
+
+/* out = o / l (bf16 or fp32, strided like q), lse = m + log(l).   Replaces ring.py:134-135
+ * and the output transpose ring.py:137.  out_dtype is RA_DTYPE_BF16 or RA_DTYPE_F32. */
+int ra_fwd_finalize(const float* o, const float* m, const float* l, void* out,
+                    int32_t out_dtype, int64_t out_stride_b, int64_t out_stride_h,
+                    int64_t out_stride_l, float* lse, int32_t B, int32_t H, int32_t Lq,
+                    int32_t D, void* stream);
+
+/* delta = rowsum(out * dout) in fp32.   Replaces _precompute_delta (ring_kernel.py:387-409)
+ * / the inline form ring.py:151.  `out` may be bf16 or fp32 (out_dtype), dout is bf16. */
+int ra_bwd_delta(const void* out, int32_t out_dtype, int64_t out_stride_b,
+                 int64_t out_stride_h, int64_t out_stride_l, const ra_tensor* dout,
+                 float* delta, int32_t B, int32_t H, int32_t Lq, int32_t D, void* stream);
+
+/* dq, dk, dv += gradients of one (query shard, key/value shard) pair, recomputed from the
+ * saved logsumexp.  Replaces bwd_block (ring_kernel.py:202-297) / _bwd_block
+ * (ring.py:140-157) and the accumulation ring.py:191-193. */
+int ra_bwd_step(const ra_bwd_step_params* p, void* stream);
+
+/* Cast an fp32 accumulator [B,H,L,D] to a strided bf16 tensor (the final dq/dk/dv in the
+ * caller's layout).   Replaces the output transposes ring.py:208-210. */
+int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t out_stride_h,
+                    int64_t out_stride_l, int32_t B, int32_t H, int32_t L, int32_t D,
+                    void* stream);
+
+/* Host-only, pure: 1 if every score of the (query shard, key/value shard) pair is masked
+ * by the positional terms of `bias` (CAUSAL / WINDOW), so that the whole ring step is an
+ * identity on the carry and may be skipped; 0 otherwise.  The reference runs such steps and
+ * lets its -inf guards nullify them (ring.py:66,69). */
+int ra_step_is_skippable(const ra_bias* bias, int32_t Lq, int32_t Lk);
+
+/* Argument checks of ra_fwd_step / ra_bwd_step without launching anything (host only). */
+int ra_fwd_step_check(const ra_fwd_step_params* p);
+int ra_bwd_step_check(const ra_bwd_step_params* p);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RING_ATTENTION_HIP_H */

@@ -1,0 +1,248 @@
+// C ABI of the ring-attention block-step library: argument validation (host only, before
+// any HIP call) and dispatch to the gfx950 kernels.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "ra_launch.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(RA_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_tensor(const char* name, const ra_tensor& t) {
+  if (!t.ptr) return fail(RA_ERR_NULL, "%s.ptr is NULL", name);
+  if (!aligned16(t.ptr)) return fail(RA_ERR_ALIGN, "%s.ptr is not 16-byte aligned", name);
+  if ((t.stride_b % 8) || (t.stride_h % 8) || (t.stride_l % 8))
+    return fail(RA_ERR_ALIGN, "%s strides must be multiples of 8 elements (16 bytes)", name);
+  return RA_OK;
+}
+
+constexpr int64_t kMaxPos = (int64_t)1 << 30;
+constexpr int kMaxLen = 1 << 24;
+constexpr int kMaxSegLen = 65536;  // tile-list capacity of the kernels (1024 tiles x 64)
+
+int check_dims(int B, int H, int Lq, int Lk, int D) {
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0)
+    return fail(RA_ERR_SHAPE, "B, H, Lq, Lk must be positive (got %d, %d, %d, %d)", B, H, Lq, Lk);
+  if (Lq > kMaxLen || Lk > kMaxLen)
+    return fail(RA_ERR_SHAPE, "shard length above %d tokens", kMaxLen);
+  if ((int64_t)B * H > (1 << 20)) return fail(RA_ERR_SHAPE, "B*H too large");
+  if (D != 64 && D != 128) return fail(RA_ERR_HEAD_DIM, "head dim %d unsupported (64 or 128)", D);
+  return RA_OK;
+}
+
+int check_bias(const ra_bias& b, int Lq, int Lk) {
+  const int known = RA_BIAS_CAUSAL | RA_BIAS_WINDOW | RA_BIAS_SEGMENT | RA_BIAS_PREFIX | RA_BIAS_ALIBI;
+  if (b.flags & ~known) return fail(RA_ERR_BIAS, "unknown bias flag bits 0x%x", b.flags & ~known);
+  if ((b.flags & RA_BIAS_WINDOW) && b.window <= 0)
+    return fail(RA_ERR_BIAS, "window must be positive (got %d)", b.window);
+  if ((b.flags & RA_BIAS_CAUSAL) && (b.flags & RA_BIAS_PREFIX))
+    return fail(RA_ERR_BIAS, "causal attention does not support a prefix mask");
+  if ((b.flags & RA_BIAS_SEGMENT) && (!b.q_segment_ids || !b.kv_segment_ids))
+    return fail(RA_ERR_NULL, "segment bias needs q_segment_ids and kv_segment_ids");
+  if ((b.flags & RA_BIAS_SEGMENT) && (Lq > kMaxSegLen || Lk > kMaxSegLen))
+    return fail(RA_ERR_SHAPE, "segment bias supports shards of at most %d tokens", kMaxSegLen);
+  if ((b.flags & RA_BIAS_PREFIX) && (!b.q_prefix || !b.kv_prefix))
+    return fail(RA_ERR_NULL, "prefix bias needs q_prefix and kv_prefix");
+  if ((b.flags & RA_BIAS_ALIBI) && !b.alibi_slopes)
+    return fail(RA_ERR_NULL, "ALiBi bias needs alibi_slopes");
+  if (b.q_offset < 0 || b.kv_offset < 0 || b.q_offset > kMaxPos || b.kv_offset > kMaxPos)
+    return fail(RA_ERR_BIAS, "token offsets must lie in [0, 2^30]");
+  return RA_OK;
+}
+
+ra::TensorArg to_arg(const ra_tensor& t) {
+  return ra::TensorArg{(const ra::bf16_t*)t.ptr, t.stride_b, t.stride_h, t.stride_l};
+}
+
+ra::BiasArgs to_bias(const ra_bias& b) {
+  ra::BiasArgs r;
+  r.flags = b.flags;
+  r.window = b.window;
+  r.q_off = (int)b.q_offset;
+  r.kv_off = (int)b.kv_offset;
+  r.q_seg = b.q_segment_ids;
+  r.kv_seg = b.kv_segment_ids;
+  r.q_seg_sb = b.q_segment_stride_b;
+  r.kv_seg_sb = b.kv_segment_stride_b;
+  r.q_pre = b.q_prefix;
+  r.kv_pre = b.kv_prefix;
+  r.q_pre_sb = b.q_prefix_stride_b;
+  r.kv_pre_sb = b.kv_prefix_stride_b;
+  r.slopes = b.alibi_slopes;
+  return r;
+}
+
+bool is_general(int flags) {
+  return (flags & (RA_BIAS_SEGMENT | RA_BIAS_PREFIX | RA_BIAS_ALIBI)) != 0;
+}
+
+constexpr float kLog2eHost = 1.4426950408889634f;
+
+}  // namespace
+
+extern "C" {
+
+int ra_version(void) { return 1000; }
+
+const char* ra_last_error(void) { return g_err; }
+
+int ra_step_is_skippable(const ra_bias* bias, int32_t Lq, int32_t Lk) {
+  if (!bias || Lq <= 0 || Lk <= 0) return 0;
+  if (bias->flags & RA_BIAS_PREFIX) return 0;
+  const int64_t qlo = bias->q_offset, qhi = bias->q_offset + Lq - 1;
+  const int64_t klo = bias->kv_offset, khi = bias->kv_offset + Lk - 1;
+  if ((bias->flags & RA_BIAS_CAUSAL) && klo > qhi) return 1;
+  if (bias->flags & RA_BIAS_WINDOW) {
+    if (qlo - khi >= bias->window) return 1;
+    if (!(bias->flags & RA_BIAS_CAUSAL) && klo - qhi >= bias->window) return 1;
+  }
+  return 0;
+}
+
+int ra_fwd_step_check(const ra_fwd_step_params* p) {
+  if (!p) return fail(RA_ERR_NULL, "params is NULL");
+  int rc = check_dims(p->B, p->H, p->Lq, p->Lk, p->D);
+  if (rc) return rc;
+  if ((rc = check_tensor("q", p->q))) return rc;
+  if ((rc = check_tensor("k", p->k))) return rc;
+  if ((rc = check_tensor("v", p->v))) return rc;
+  if (!p->o || !p->m || !p->l) return fail(RA_ERR_NULL, "carry pointer (o, m or l) is NULL");
+  if (!aligned16(p->o)) return fail(RA_ERR_ALIGN, "o is not 16-byte aligned");
+  if (!(p->sm_scale == p->sm_scale) || p->sm_scale == 0.f)
+    return fail(RA_ERR_SHAPE, "sm_scale must be a non-zero number");
+  return check_bias(p->bias, p->Lq, p->Lk);
+}
+
+int ra_bwd_step_check(const ra_bwd_step_params* p) {
+  if (!p) return fail(RA_ERR_NULL, "params is NULL");
+  int rc = check_dims(p->B, p->H, p->Lq, p->Lk, p->D);
+  if (rc) return rc;
+  if ((rc = check_tensor("q", p->q))) return rc;
+  if ((rc = check_tensor("k", p->k))) return rc;
+  if ((rc = check_tensor("v", p->v))) return rc;
+  if ((rc = check_tensor("dout", p->dout))) return rc;
+  if (!p->lse || !p->delta) return fail(RA_ERR_NULL, "lse or delta is NULL");
+  if (!p->dq || !p->dk || !p->dv) return fail(RA_ERR_NULL, "gradient accumulator (dq, dk or dv) is NULL");
+  if (!aligned16(p->dq) || !aligned16(p->dk) || !aligned16(p->dv))
+    return fail(RA_ERR_ALIGN, "gradient accumulators must be 16-byte aligned");
+  if (!(p->sm_scale == p->sm_scale) || p->sm_scale == 0.f)
+    return fail(RA_ERR_SHAPE, "sm_scale must be a non-zero number");
+  return check_bias(p->bias, p->Lq, p->Lk);
+}
+
+int ra_fwd_init(float* o, float* m, float* l, int32_t B, int32_t H, int32_t Lq, int32_t D, void* stream) {
+  if (!o || !m || !l) return fail(RA_ERR_NULL, "carry pointer (o, m or l) is NULL");
+  int rc = check_dims(B, H, Lq, 1, D);
+  if (rc) return rc;
+  hipError_t e = ra::launch_fwd_init(o, m, l, (long long)B * H * Lq, D, (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_init launch");
+}
+
+int ra_fwd_step(const ra_fwd_step_params* p, void* stream) {
+  int rc = ra_fwd_step_check(p);
+  if (rc) return rc;
+  if (ra_step_is_skippable(&p->bias, p->Lq, p->Lk)) return RA_OK;  // identity on the carry
+  ra::FwdArgs a;
+  a.q = to_arg(p->q);
+  a.k = to_arg(p->k);
+  a.v = to_arg(p->v);
+  a.o = p->o;
+  a.m = p->m;
+  a.l = p->l;
+  a.B = p->B;
+  a.H = p->H;
+  a.Lq = p->Lq;
+  a.Lk = p->Lk;
+  a.scale2 = p->sm_scale * kLog2eHost;
+  a.bias = to_bias(p->bias);
+  hipError_t e = ra::launch_fwd_step(a, p->D, is_general(p->bias.flags), (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_step launch");
+}
+
+int ra_fwd_finalize(const float* o, const float* m, const float* l, void* out, int32_t out_dtype,
+                    int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l, float* lse,
+                    int32_t B, int32_t H, int32_t Lq, int32_t D, void* stream) {
+  if (!o || !m || !l || !out || !lse) return fail(RA_ERR_NULL, "ra_fwd_finalize: NULL pointer");
+  int rc = check_dims(B, H, Lq, 1, D);
+  if (rc) return rc;
+  if (out_dtype != RA_DTYPE_BF16 && out_dtype != RA_DTYPE_F32)
+    return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
+  if ((out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
+    return fail(RA_ERR_ALIGN, "out strides must be multiples of 4 elements");
+  hipError_t e = ra::launch_fwd_finalize(o, m, l, out, out_dtype == RA_DTYPE_F32, out_stride_b,
+                                         out_stride_h, out_stride_l, lse, B, H, Lq, D,
+                                         (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_finalize launch");
+}
+
+int ra_bwd_delta(const void* out, int32_t out_dtype, int64_t out_stride_b, int64_t out_stride_h,
+                 int64_t out_stride_l, const ra_tensor* dout, float* delta, int32_t B, int32_t H,
+                 int32_t Lq, int32_t D, void* stream) {
+  if (!out || !dout || !delta) return fail(RA_ERR_NULL, "ra_bwd_delta: NULL pointer");
+  int rc = check_dims(B, H, Lq, 1, D);
+  if (rc) return rc;
+  if ((rc = check_tensor("dout", *dout))) return rc;
+  if (out_dtype != RA_DTYPE_BF16 && out_dtype != RA_DTYPE_F32)
+    return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
+  if (!aligned16(out) || (out_stride_b % 8) || (out_stride_h % 8) || (out_stride_l % 8))
+    return fail(RA_ERR_ALIGN, "out must be 16-byte aligned with strides that are multiples of 8");
+  hipError_t e = ra::launch_bwd_delta(out, out_dtype == RA_DTYPE_F32, out_stride_b, out_stride_h,
+                                      out_stride_l, to_arg(*dout), delta, B, H, Lq, D,
+                                      (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_delta launch");
+}
+
+int ra_bwd_step(const ra_bwd_step_params* p, void* stream) {
+  int rc = ra_bwd_step_check(p);
+  if (rc) return rc;
+  if (ra_step_is_skippable(&p->bias, p->Lq, p->Lk)) return RA_OK;  // contributes nothing
+  ra::BwdArgs a;
+  a.q = to_arg(p->q);
+  a.k = to_arg(p->k);
+  a.v = to_arg(p->v);
+  a.dout = to_arg(p->dout);
+  a.lse = p->lse;
+  a.delta = p->delta;
+  a.dq = p->dq;
+  a.dk = p->dk;
+  a.dv = p->dv;
+  a.B = p->B;
+  a.H = p->H;
+  a.Lq = p->Lq;
+  a.Lk = p->Lk;
+  a.scale2 = p->sm_scale * kLog2eHost;
+  a.sm_scale = p->sm_scale;
+  a.bias = to_bias(p->bias);
+  hipError_t e = ra::launch_bwd_step(a, p->D, is_general(p->bias.flags), (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_step launch");
+}
+
+int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t out_stride_h,
+                    int64_t out_stride_l, int32_t B, int32_t H, int32_t L, int32_t D, void* stream) {
+  if (!acc || !out) return fail(RA_ERR_NULL, "ra_bwd_finalize: NULL pointer");
+  int rc = check_dims(B, H, L, 1, D);
+  if (rc) return rc;
+  if ((out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
+    return fail(RA_ERR_ALIGN, "out strides must be multiples of 4 elements");
+  hipError_t e = ra::launch_bwd_finalize(acc, out, out_stride_b, out_stride_h, out_stride_l, B, H, L,
+                                         D, (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_finalize launch");
+}
+
+}  // extern "C"

@@ -1,0 +1,270 @@
+// Shared device-side helpers for the gfx950 ring-attention kernels: vector types, the
+// bank-conflict-free LDS tile layout, global->LDS tile staging, MFMA operand fetches and
+// the per-tile bias functor.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/ring_attention_hip.h"
+
+namespace ra {
+
+typedef __bf16 bf16_t;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+#define RA_DEV __device__ __forceinline__
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+#define RA_NEG_INF (-__builtin_inff())
+
+// Device-side view of ra_bias for one (batch, head): pointers already moved to the batch
+// row, the ALiBi slope already multiplied by log2(e).
+struct BiasArgs {
+  int flags;
+  int window;
+  int q_off;   // position of local query 0
+  int kv_off;  // position of local key 0
+  const int* q_seg;
+  const int* kv_seg;
+  long long q_seg_sb, kv_seg_sb;
+  const int* q_pre;
+  const int* kv_pre;
+  long long q_pre_sb, kv_pre_sb;
+  const float* slopes;
+};
+
+struct TensorArg {
+  const bf16_t* ptr;
+  long long sb, sh, sl;
+};
+
+// ---------------------------------------------------------------------------------------
+// wave-level helpers (wave64)
+// ---------------------------------------------------------------------------------------
+// Value held by the partner lane (lane ^ 32) combined with the own one.
+RA_DEV float half_max(float x) {
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+RA_DEV float half_sum(float x) {
+  unsigned u = __float_as_uint(x);
+  auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+RA_DEV int wave_min(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+  return v;
+}
+RA_DEV int wave_max(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
+RA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---------------------------------------------------------------------------------------
+// LDS tile layout.  A tile is [rows][D] bf16, row-major, and the 16-byte chunks of a row
+// are permuted by an XOR with a function of the row so that BOTH access patterns the
+// kernels use hit 64 distinct banks:
+//   * "natural" MFMA operand fetch: 16 consecutive rows, the same chunk, one b128 per lane;
+//   * transposing fetch (ds_read_b64_tr_b16): 4 consecutive rows x 64 contiguous bytes.
+// ---------------------------------------------------------------------------------------
+template <int D>
+RA_DEV int tile_off(int row, int chunk) {
+  if (D == 128) {
+    int f = ((row & 3) << 2) | ((row >> 2) & 3);
+    return row * 256 + ((chunk ^ f) << 4);
+  } else {
+    int f = (row >> 1) & 7;
+    return row * 128 + ((chunk ^ f) << 4);
+  }
+}
+
+typedef __attribute__((address_space(3))) char lds_char;
+
+// A/B operand of v_mfma_f32_32x32x16_bf16 taken along the contiguous (head-dim) axis:
+// lane holds row (row0 + lane%32), elements [16*ks + 8*(lane/32), +8).
+template <int D>
+RA_DEV bf16x8 frag_nat(const char* tile, int row, int ks, int g) {
+  return *(const bf16x8*)(tile + tile_off<D>(row, 2 * ks + g));
+}
+
+// Operand taken ACROSS rows (the contraction index is the tile's row index): lane gets,
+// for column (col0 + lane%32), the 8 rows  rbase + {0..3}  and  rbase + 8 + {0..3}  where
+// rbase = row16 + 4*(lane/32).  That is the row set an accumulator lane of the 32x32
+// MFMA holds in registers 8*ks .. 8*ks+7, so the two operands pair up element by element.
+template <int D>
+RA_DEV bf16x8 frag_tr(const char* tile, int row16, int col0, int lane) {
+  const int j = lane & 15;
+  const int row = row16 + 4 * (lane >> 5) + (j >> 2);
+  const int col = col0 + 16 * ((lane >> 4) & 1) + 4 * (j & 3);  // element index
+  const int chunk = col >> 3;
+  const int sub = (col & 4) << 1;  // byte offset inside the chunk (0 or 8)
+  const lds_char* p0 = (const lds_char*)(tile + tile_off<D>(row, chunk) + sub);
+  const lds_char* p1 = (const lds_char*)(tile + tile_off<D>(row + 8, chunk) + sub);
+  bf16x4 a = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p0);
+  bf16x4 b = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p1);
+  return __builtin_shufflevector(a, b, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// Global -> registers -> LDS staging of a [ROWS][D] bf16 tile by NT threads.
+template <int D, int ROWS, int NT>
+struct TileStage {
+  static constexpr int CPR = D / 8;  // 16-byte chunks per row
+  static constexpr int TOTAL = ROWS * CPR;
+  static constexpr int N = (TOTAL + NT - 1) / NT;
+  u32x4 r[N];
+  // rows row0 .. row0+ROWS-1 of a [L][D] matrix with row stride sl; rows >= L are clamped
+  RA_DEV void load(const bf16_t* base, long long sl, int row0, int L, int tid) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int idx = tid + i * NT;
+      if (TOTAL % NT == 0 || idx < TOTAL) {
+        int row = idx / CPR, c = idx % CPR;
+        int gr = min(row0 + row, L - 1);
+        r[i] = *(const u32x4*)(base + (long long)gr * sl + c * 8);
+      }
+    }
+  }
+  RA_DEV void store(char* tile, int tid) const {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      int idx = tid + i * NT;
+      if (TOTAL % NT == 0 || idx < TOTAL) {
+        int row = idx / CPR, c = idx % CPR;
+        *(u32x4*)(tile + tile_off<D>(row, c)) = r[i];
+      }
+    }
+  }
+};
+
+RA_DEV bf16x8 pack8(const f32x16& p, int base) {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) r[i] = (bf16_t)p[base + i];
+  return r;
+}
+
+// ---------------------------------------------------------------------------------------
+// Bias functor on one 32x32 accumulator block.
+// The accumulator lane owns ONE index on the "fixed" side (lane%32) and 16 indices on the
+// "varying" side: var0 + 8*(r/4) + (r%4), r = 0..15 (var0 already includes 4*(lane/32)).
+// QFIXED = true : fixed side is the query, varying side the keys (S^T blocks);
+// QFIXED = false: fixed side is the key, varying side the queries (S blocks).
+// `rel0` = q_pos - kv_pos for r = 0.  fixed_seg / fixed_pre are the lane's own id values,
+// var_seg / var_pre point at the LDS copies of the varying side's ids for var0.
+// ---------------------------------------------------------------------------------------
+struct TileBias {
+  int flags;     // terms that must be evaluated for this block
+  int window;
+  float slope2;  // ALiBi slope * log2(e)
+  int var_limit; // varying-side indices >= var_limit (relative to var0) are out of range
+};
+
+template <bool QFIXED>
+RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, int fixed_pre,
+                       const int* var_seg, const int* var_pre) {
+#pragma unroll
+  for (int bb = 0; bb < 4; ++bb) {
+    i32x4 vs = {0, 0, 0, 0}, vp = {0, 0, 0, 0};
+    if (tb.flags & RA_BIAS_SEGMENT) vs = *(const i32x4*)(var_seg + 8 * bb);
+    if (tb.flags & RA_BIAS_PREFIX) vp = *(const i32x4*)(var_pre + 8 * bb);
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int r = 4 * bb + c;
+      const int off = 8 * bb + c;
+      // moving along the varying side: keys advance -> rel decreases; queries advance -> rel increases
+      const int rel = QFIXED ? rel0 - off : rel0 + off;
+      float x = t[r];
+      if (tb.flags & RA_BIAS_ALIBI) x = fmaf(fabsf((float)rel), -tb.slope2, x);
+      bool msk = off >= tb.var_limit;
+      if (tb.flags & RA_BIAS_CAUSAL) msk |= rel < 0;
+      if (tb.flags & RA_BIAS_WINDOW) {
+        msk |= rel >= tb.window;
+        if (!(tb.flags & RA_BIAS_CAUSAL)) msk |= -rel >= tb.window;
+      }
+      if (tb.flags & RA_BIAS_SEGMENT) msk |= vs[c] != fixed_seg;
+      if (tb.flags & RA_BIAS_PREFIX) msk |= !(((vp[c] & fixed_pre) != 0) | (rel >= 0));
+      t[r] = msk ? RA_NEG_INF : x;
+    }
+  }
+}
+
+// Positional classification of a rectangle of scores: queries [qlo, qhi], keys [klo, khi]
+// (global positions, inclusive).  Returns bit 0 = every score masked, bit 1 = some score may
+// be masked (the elementwise test is needed).
+RA_DEV int classify_pos(int flags, int window, int qlo, int qhi, int klo, int khi) {
+  bool all = false, some = false;
+  if (flags & RA_BIAS_CAUSAL) {
+    all |= klo > qhi;
+    some |= khi > qlo;
+  }
+  if (flags & RA_BIAS_WINDOW) {
+    all |= (qlo - khi) >= window;
+    some |= (qhi - klo) >= window;
+    if (!(flags & RA_BIAS_CAUSAL)) {
+      all |= (klo - qhi) >= window;
+      some |= (khi - qlo) >= window;
+    }
+  }
+  return (all ? 1 : 0) | (some ? 2 : 0);
+}
+
+RA_DEV int floor_div(int a, int b) { return (a >= 0) ? a / b : -((-a + b - 1) / b); }
+RA_DEV int ceil_div(int a, int b) { return -floor_div(-a, b); }
+
+// Range [lo, hi) of T-sized tiles on the key side that can hold an unmasked score for
+// queries at positions [qlo, qhi]; keys of tile j are at positions kv_off + T*j + [0, T).
+RA_DEV void key_tile_range(int flags, int window, int qlo, int qhi, int kv_off, int ntiles, int T,
+                           int& lo, int& hi) {
+  lo = 0;
+  hi = ntiles;
+  if (flags & RA_BIAS_PREFIX) return;
+  if (flags & RA_BIAS_CAUSAL) hi = min(hi, floor_div(qhi - kv_off, T) + 1);
+  if (flags & RA_BIAS_WINDOW) {
+    lo = max(lo, ceil_div(qlo - window + 1 - (T - 1) - kv_off, T));
+    if (!(flags & RA_BIAS_CAUSAL)) hi = min(hi, floor_div(qhi + window - 1 - kv_off, T) + 1);
+  }
+  hi = max(hi, 0);
+  lo = min(max(lo, 0), hi);
+}
+
+// Same for the query side: tiles of queries that can see keys at positions [klo, khi].
+RA_DEV void query_tile_range(int flags, int window, int klo, int khi, int q_off, int ntiles, int T,
+                             int& lo, int& hi) {
+  lo = 0;
+  hi = ntiles;
+  if (flags & RA_BIAS_PREFIX) return;
+  if (flags & RA_BIAS_CAUSAL) lo = max(lo, ceil_div(klo - (T - 1) - q_off, T));
+  if (flags & RA_BIAS_WINDOW) {
+    hi = min(hi, floor_div(khi + window - 1 - q_off, T) + 1);
+    if (!(flags & RA_BIAS_CAUSAL)) lo = max(lo, ceil_div(klo - window + 1 - (T - 1) - q_off, T));
+  }
+  hi = max(hi, 0);
+  lo = min(max(lo, 0), hi);
+}
+
+// Decode the flat workgroup id into (batch*head index, tile index).  Workgroups are handed
+// to the 8 XCDs round-robin, each XCD has its own L2: keep all tiles of one head on one
+// XCD so they share the head's K/V (or Q/dO) stream, and start with the last tile, which
+// has the most work under a causal mask.
+RA_DEV void decode_block(int bid, int BH, int ntile, int& hh, int& tile) {
+  if ((BH & 7) == 0) {
+    int xcd = bid & 7, slot = bid >> 3;
+    hh = (slot / ntile) * 8 + xcd;
+    tile = ntile - 1 - (slot % ntile);
+  } else {
+    hh = bid / ntile;
+    tile = ntile - 1 - (bid % ntile);
+  }
+}
+
+}  // namespace ra

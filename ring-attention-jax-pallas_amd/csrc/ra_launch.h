@@ -1,0 +1,43 @@
+// Kernel argument blocks and host launchers shared between the kernel translation units
+// and the C ABI.
+#pragma once
+#include "ra_common.h"
+
+namespace ra {
+
+struct FwdArgs {
+  TensorArg q, k, v;
+  float* o;
+  float* m;
+  float* l;
+  int B, H, Lq, Lk;
+  float scale2;  // sm_scale * log2(e)
+  BiasArgs bias;
+};
+
+struct BwdArgs {
+  TensorArg q, k, v, dout;
+  const float* lse;
+  const float* delta;
+  float* dq;
+  float* dk;
+  float* dv;
+  int B, H, Lq, Lk;
+  float scale2;    // sm_scale * log2(e)
+  float sm_scale;
+  BiasArgs bias;
+};
+
+hipError_t launch_fwd_step(const FwdArgs& a, int D, bool general, hipStream_t stream);
+hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream);
+hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, void* out, int out_f32,
+                               long long sb, long long sh, long long sl, float* lse, int B, int H,
+                               int Lq, int D, hipStream_t stream);
+hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long long sh, long long sl,
+                            TensorArg dout, float* delta, int B, int H, int Lq, int D,
+                            hipStream_t stream);
+hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, hipStream_t stream);
+hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl,
+                               int B, int H, int L, int D, hipStream_t stream);
+
+}  // namespace ra

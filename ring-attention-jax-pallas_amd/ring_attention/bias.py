@@ -1,0 +1,156 @@
+"""Declarative attention-bias terms: the device-side form of the reference's ``bias_fn``.
+
+The reference lets the user pass any ``bias_fn(**bias_q_kwargs, **bias_kv_kwargs)`` that
+returns a dense additive ``[b, h, lq, lk]`` block per ring step (ring.py:107,186).  A dense
+block is 1 GiB per head at 16k x 16k, so here a bias is DESCRIBED by a ``BiasFn`` object and
+evaluated inside the kernels, tile by tile, from token positions and per-token id arrays.
+Terms add up exactly as additive biases do (0 / -inf masks and finite ALiBi penalties):
+
+    bias_fn = causal_bias() + segment_bias()              # ring.py:388-397
+    bias_fn = prefix_lm_bias() + segment_bias()           # ring.py:399-406
+    bias_fn = sliding_window_bias(4096)                   # causal window
+    bias_fn = segment_bias() + alibi_bias(slopes)
+
+The per-token arrays keep the reference's kwarg names (ring.py:411-420):
+``q_segment_ids`` / ``kv_segment_ids``, ``q_positions`` / ``kv_positions``,
+``q_prefix_mask`` / ``kv_prefix_mask``; the q-side ones go into ``bias_q_kwargs`` and the
+kv-side ones into ``bias_kv_kwargs``.  Positions are optional: when absent a token's
+position is its index in the global sequence; when given they must be consecutive inside
+every shard (the kernels take one offset per shard).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, replace
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+
+@dataclass(frozen=True)
+class BiasFn:
+    causal: bool = False
+    window: Optional[int] = None
+    segments: bool = False
+    prefix: bool = False
+    alibi_slopes: Optional[torch.Tensor] = None  # [H] float32
+
+    def __add__(self, other: "BiasFn") -> "BiasFn":
+        if not isinstance(other, BiasFn):
+            return NotImplemented
+        if self.window is not None and other.window is not None:
+            window = min(self.window, other.window)
+        else:
+            window = self.window if self.window is not None else other.window
+        if self.alibi_slopes is not None and other.alibi_slopes is not None:
+            slopes = self.alibi_slopes + other.alibi_slopes
+        else:
+            slopes = self.alibi_slopes if self.alibi_slopes is not None else other.alibi_slopes
+        out = BiasFn(self.causal or other.causal, window, self.segments or other.segments,
+                     self.prefix or other.prefix, slopes)
+        out.validate()
+        return out
+
+    def validate(self) -> None:
+        # same rule as ring_self_attention's asserts (ring.py:368-374)
+        if self.causal and self.prefix:
+            raise ValueError("causal attention does not support prefix_mask")
+        if self.window is not None and self.window <= 0:
+            raise ValueError("window must be positive")
+
+    @property
+    def flags(self) -> int:
+        f = 0
+        if self.causal:
+            f |= _lib.RA_BIAS_CAUSAL
+        if self.window is not None:
+            f |= _lib.RA_BIAS_WINDOW
+        if self.segments:
+            f |= _lib.RA_BIAS_SEGMENT
+        if self.prefix:
+            f |= _lib.RA_BIAS_PREFIX
+        if self.alibi_slopes is not None:
+            f |= _lib.RA_BIAS_ALIBI
+        return f
+
+    @property
+    def needs_positions(self) -> bool:
+        return self.causal or self.prefix or self.window is not None or self.alibi_slopes is not None
+
+
+def causal_bias() -> BiasFn:
+    """0 where kv_position <= q_position, -inf elsewhere (ring.py:393-397)."""
+    return BiasFn(causal=True)
+
+
+def sliding_window_bias(window: int, causal: bool = True) -> BiasFn:
+    """0 where 0 <= q_pos - kv_pos < window (or |q_pos - kv_pos| < window if not causal)."""
+    b = BiasFn(causal=causal, window=int(window))
+    b.validate()
+    return b
+
+
+def segment_bias() -> BiasFn:
+    """0 where q_segment_ids == kv_segment_ids, -inf elsewhere (ring.py:388-391)."""
+    return BiasFn(segments=True)
+
+
+def prefix_lm_bias() -> BiasFn:
+    """0 where (q_prefix_mask & kv_prefix_mask) | kv_pos <= q_pos (ring.py:399-406)."""
+    return BiasFn(prefix=True)
+
+
+def alibi_bias(slopes) -> BiasFn:
+    """-slopes[h] * |q_pos - kv_pos| added to the scaled scores of head h."""
+    return BiasFn(alibi_slopes=torch.as_tensor(slopes, dtype=torch.float32))
+
+
+def alibi_slopes(num_heads: int) -> torch.Tensor:
+    """The geometric slope family 2^(-8 h / H), h = 1..H."""
+    return torch.tensor([2.0 ** (-8.0 * (h + 1) / num_heads) for h in range(num_heads)],
+                        dtype=torch.float32)
+
+
+@dataclass
+class BlockBias:
+    """A BiasFn bound to ONE (query shard, key/value shard) pair: what ``bias_fn(...)``
+    returns for a ring step in the reference, in un-materialised form."""
+    fn: BiasFn
+    q_offset: int = 0
+    kv_offset: int = 0
+    q_segment_ids: Optional[torch.Tensor] = None   # int32 [b, lq]
+    kv_segment_ids: Optional[torch.Tensor] = None  # int32 [b, lk]
+    q_prefix_mask: Optional[torch.Tensor] = None   # int32 [b, lq]
+    kv_prefix_mask: Optional[torch.Tensor] = None  # int32 [b, lk]
+
+    def to_struct(self, device) -> "_lib.RaBias":
+        s = _lib.RaBias()
+        fn = self.fn
+        s.flags = fn.flags
+        s.window = fn.window or 0
+        s.q_offset = int(self.q_offset)
+        s.kv_offset = int(self.kv_offset)
+        self._keep = []
+
+        def ids(t, name):
+            if t is None:
+                raise ValueError(f"bias needs {name}")
+            if t.dtype != torch.int32 or t.stride(-1) != 1 or t.device != device:
+                raise ValueError(f"{name} must be an int32 tensor on {device} with unit inner stride")
+            self._keep.append(t)
+            return t.data_ptr(), t.stride(0)
+
+        if fn.segments:
+            s.q_segment_ids, s.q_segment_stride_b = ids(self.q_segment_ids, "q_segment_ids")
+            s.kv_segment_ids, s.kv_segment_stride_b = ids(self.kv_segment_ids, "kv_segment_ids")
+        if fn.prefix:
+            s.q_prefix, s.q_prefix_stride_b = ids(self.q_prefix_mask, "q_prefix_mask")
+            s.kv_prefix, s.kv_prefix_stride_b = ids(self.kv_prefix_mask, "kv_prefix_mask")
+        if fn.alibi_slopes is not None:
+            sl = fn.alibi_slopes
+            if sl.device != device:
+                raise ValueError("alibi slopes must be moved to the compute device first")
+            self._keep.append(sl)
+            s.alibi_slopes = sl.data_ptr()
+        return s

@@ -1,0 +1,428 @@
+"""Ring attention on one MI355X: the reference's call surface over the HIP block-step kernels.
+
+Public names follow the reference (``ring.py:246`` ``ring_attention``, ``ring.py:328``
+``ring_self_attention``; block functions ``ring_kernel.py:123`` ``fwd_block`` and
+``ring_kernel.py:202`` ``bwd_block``).  What differs, and why:
+
+* There is one GPU and no mesh.  ``q, k, v`` are the GLOBAL ``[b, S, h, d]`` arrays and
+  ``axis_name`` carries the ring size (``RingAxis("sp", 8)`` or just ``8``).  The ring is
+  emulated: the arrays are cut into ``size`` shards along the sequence; "device" r keeps
+  query shard r and its fp32 ``(o, m, l)`` carry, and at step t meets the key/value shard
+  that started on device ``(r - t) mod size`` - the order ``ppermute`` produces in
+  ``ring.py:51-55,120``.  In the backward pass the query side travels instead
+  (``ring.py:195``).  The result is what ``shard_map(ring_attention)`` returns for the
+  global arrays.
+* ``bias_fn`` is a declarative ``BiasFn`` (see ``bias.py``) evaluated inside the kernels;
+  ring steps and score tiles that are entirely masked are skipped.
+* Compute is bf16 on the matrix cores with fp32 carries; other input dtypes are cast on
+  entry and the result is cast back.  Head dims other than 64/128 are zero-padded.
+
+Everything runs through ``libringattn_hip.so``; if it is missing the import of this module
+succeeds but every call raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from dataclasses import dataclass
+from typing import Optional, Union
+
+import torch
+
+from . import _lib
+from .bias import BiasFn, BlockBias
+
+_IMPLS = ("hip", "pallas")  # "pallas" is accepted as an alias: the fused-kernel choice
+
+
+@dataclass(frozen=True)
+class RingAxis:
+    """Stands in for the mesh axis the reference shards sequences over."""
+    name: str
+    size: int
+
+
+def _axis_size(axis_name) -> int:
+    if isinstance(axis_name, RingAxis):
+        return axis_name.size
+    if isinstance(axis_name, int):
+        return axis_name
+    if isinstance(axis_name, (tuple, list)) and len(axis_name) == 2:
+        return int(axis_name[1])
+    raise TypeError("axis_name must be a RingAxis, an int ring size or a (name, size) pair")
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require_gpu(t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise RuntimeError("ring_attention runs on the GPU only: tensors must live on a HIP device "
+                           "(there is no CPU fallback)")
+
+
+def _view_bhld(t: torch.Tensor) -> _lib.RaTensor:
+    """RaTensor for a tensor indexed [b, h, l, d] (any strides, d contiguous)."""
+    return _lib.RaTensor(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
+    """bf16, unit inner stride, 16-byte aligned rows."""
+    if t.dtype != torch.bfloat16:
+        t = t.to(torch.bfloat16)
+    ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    return t if ok else t.contiguous()
+
+
+# --------------------------------------------------------------------------------------
+# block-level API (one ring step)
+# --------------------------------------------------------------------------------------
+def _bias_struct(bias: Optional[BlockBias], device) -> _lib.RaBias:
+    if bias is None:
+        return _lib.RaBias()
+    return bias.to_struct(device)
+
+
+def fwd_block(q, k, v, bias: Optional[BlockBias], o, m, l, sm_scale: float):
+    """One ring step of the forward pass, in place on the fp32 carry.
+
+    Same contract as the reference's ``fwd_block`` (ring_kernel.py:123-199): ``q`` is
+    ``[b, h, lq, d]``, ``k``/``v`` are ``[b, h, lk, d]`` (bf16, any batch/head/length strides),
+    ``o`` ``[b, h, lq, d]`` is the unnormalised output and ``m``/``l`` ``[b, h, lq]`` the
+    running max / sum (fp32, contiguous).  ``bias`` describes the block's additive bias.
+    Returns ``(o, m, l)`` (the same tensors, updated)."""
+    _require_gpu(q)
+    lib = _lib.load()
+    B, H, Lq, D = q.shape
+    p = _lib.RaFwdStepParams()
+    p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
+    p.sm_scale = float(sm_scale)
+    p.q, p.k, p.v = _view_bhld(q), _view_bhld(k), _view_bhld(v)
+    for t_ in (o, m, l):
+        if t_.dtype != torch.float32 or not t_.is_contiguous():
+            raise ValueError("o, m, l carries must be contiguous float32 tensors")
+    p.o, p.m, p.l = o.data_ptr(), m.data_ptr(), l.data_ptr()
+    p.bias = _bias_struct(bias, q.device)
+    _lib.check("ra_fwd_step", lib.ra_fwd_step(C.byref(p), _stream()))
+    return o, m, l
+
+
+def init_carry(batch, heads, q_len, dim, device):
+    """Fresh carry o = 0, l = 0, m = -inf (ring.py:124-126), fp32."""
+    lib = _lib.load()
+    o = torch.empty((batch, heads, q_len, dim), dtype=torch.float32, device=device)
+    m = torch.empty((batch, heads, q_len), dtype=torch.float32, device=device)
+    l = torch.empty((batch, heads, q_len), dtype=torch.float32, device=device)
+    reset_carry(o, m, l)
+    return o, m, l
+
+
+def reset_carry(o, m, l):
+    lib = _lib.load()
+    B, H, Lq, D = o.shape
+    _lib.check("ra_fwd_init", lib.ra_fwd_init(o.data_ptr(), m.data_ptr(), l.data_ptr(), B, H, Lq, D,
+                                              _stream()))
+
+
+def finalize_carry(o, m, l, out, lse):
+    """out = o / l written into ``out`` ([b, h, lq, d] view, bf16 or fp32), lse = m + log l
+    (ring.py:134-135)."""
+    lib = _lib.load()
+    B, H, Lq, D = o.shape
+    dt = {torch.bfloat16: _lib.RA_DTYPE_BF16, torch.float32: _lib.RA_DTYPE_F32}[out.dtype]
+    _lib.check("ra_fwd_finalize", lib.ra_fwd_finalize(
+        o.data_ptr(), m.data_ptr(), l.data_ptr(), out.data_ptr(), dt, out.stride(0), out.stride(1),
+        out.stride(2), lse.data_ptr(), B, H, Lq, D, _stream()))
+
+
+def precompute_delta(out, do, delta=None):
+    """delta = rowsum(out * do) in fp32 (ring_kernel.py:387-409).  ``out`` (bf16 or fp32) and
+    ``do`` (bf16) are ``[b, h, l, d]`` views; returns ``[b, h, l]``."""
+    _require_gpu(out)
+    lib = _lib.load()
+    B, H, L, D = out.shape
+    if delta is None:
+        delta = torch.empty((B, H, L), dtype=torch.float32, device=out.device)
+    dt = {torch.bfloat16: _lib.RA_DTYPE_BF16, torch.float32: _lib.RA_DTYPE_F32}[out.dtype]
+    do_t = _view_bhld(do)
+    _lib.check("ra_bwd_delta", lib.ra_bwd_delta(out.data_ptr(), dt, out.stride(0), out.stride(1),
+                                                out.stride(2), C.byref(do_t), delta.data_ptr(), B, H,
+                                                L, D, _stream()))
+    return delta
+
+
+def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale):
+    lib = _lib.load()
+    B, H, Lq, D = q.shape
+    p = _lib.RaBwdStepParams()
+    p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
+    p.sm_scale = float(sm_scale)
+    p.q, p.k, p.v, p.dout = _view_bhld(q), _view_bhld(k), _view_bhld(v), _view_bhld(do)
+    p.lse, p.delta = lse.data_ptr(), delta.data_ptr()
+    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    p.bias = _bias_struct(bias, q.device)
+    _lib.check("ra_bwd_step", lib.ra_bwd_step(C.byref(p), _stream()))
+
+
+def bwd_block(q, k, v, bias: Optional[BlockBias], o, L, do, sm_scale: float):
+    """Gradients of one (query block, key/value block) pair, as the reference's
+    ``bwd_block`` (ring_kernel.py:202-297): all tensors ``[b, h, l, d]``, ``o`` the normalised
+    forward output, ``L`` the logsumexp ``[b, h, lq]``.  Returns fp32 ``(dq, dk, dv)``."""
+    _require_gpu(q)
+    delta = precompute_delta(o, do)
+    dq = torch.zeros(q.shape, dtype=torch.float32, device=q.device)
+    dk = torch.zeros(k.shape, dtype=torch.float32, device=q.device)
+    dv = torch.zeros(v.shape, dtype=torch.float32, device=q.device)
+    _bwd_step(q, k, v, do, L.contiguous(), delta, dq, dk, dv, bias, sm_scale)
+    return dq, dk, dv
+
+
+def _finalize_grad(acc, out):
+    lib = _lib.load()
+    B, H, L, D = acc.shape
+    _lib.check("ra_bwd_finalize", lib.ra_bwd_finalize(acc.data_ptr(), out.data_ptr(), out.stride(0),
+                                                      out.stride(1), out.stride(2), B, H, L, D,
+                                                      _stream()))
+
+
+# --------------------------------------------------------------------------------------
+# emulated ring
+# --------------------------------------------------------------------------------------
+class _RingPlan:
+    """Shard bookkeeping shared by the forward and backward loops."""
+
+    def __init__(self, q, k, n, fn: Optional[BiasFn], q_kwargs, kv_kwargs):
+        self.n = n
+        self.B, Sq, self.H, self.D = q.shape
+        Sk = k.shape[1]
+        if Sq % n or Sk % n:
+            raise ValueError(f"sequence lengths ({Sq}, {Sk}) must be divisible by the ring size {n}")
+        self.Lq, self.Lk = Sq // n, Sk // n
+        self.fn = fn
+        dev = q.device
+        q_kwargs = dict(q_kwargs or {})
+        kv_kwargs = dict(kv_kwargs or {})
+        known_q = {"q_segment_ids", "q_positions", "q_prefix_mask"}
+        known_kv = {"kv_segment_ids", "kv_positions", "kv_prefix_mask"}
+        for name in list(q_kwargs) + list(kv_kwargs):
+            if name not in known_q | known_kv:
+                raise ValueError(f"unknown bias kwarg {name!r}; expected one of "
+                                 f"{sorted(known_q | known_kv)}")
+        if fn is None and any(v is not None for v in list(q_kwargs.values()) + list(kv_kwargs.values())):
+            raise ValueError("bias kwargs were given without a bias_fn")
+
+        def ids(t, S, name):
+            if t is None:
+                return None
+            if tuple(t.shape) != (self.B, S):
+                raise ValueError(f"{name} must have shape {(self.B, S)}, got {tuple(t.shape)}")
+            return t.to(device=dev, dtype=torch.int32).contiguous()
+
+        self.q_seg = self.kv_seg = self.q_pre = self.kv_pre = None
+        self.q_off = [r * self.Lq for r in range(n)]
+        self.kv_off = [r * self.Lk for r in range(n)]
+        if fn is not None:
+            fn.validate()
+            if fn.segments:
+                self.q_seg = ids(q_kwargs.get("q_segment_ids"), Sq, "q_segment_ids")
+                self.kv_seg = ids(kv_kwargs.get("kv_segment_ids"), Sk, "kv_segment_ids")
+                if self.q_seg is None or self.kv_seg is None:
+                    raise ValueError("segment bias needs q_segment_ids and kv_segment_ids")
+            if fn.prefix:
+                self.q_pre = ids(q_kwargs.get("q_prefix_mask"), Sq, "q_prefix_mask")
+                self.kv_pre = ids(kv_kwargs.get("kv_prefix_mask"), Sk, "kv_prefix_mask")
+                if self.q_pre is None or self.kv_pre is None:
+                    raise ValueError("prefix bias needs q_prefix_mask and kv_prefix_mask")
+            if fn.needs_positions:
+                qp, kp = q_kwargs.get("q_positions"), kv_kwargs.get("kv_positions")
+                if qp is not None:
+                    self.q_off = self._offsets(qp, Sq, self.Lq, "q_positions")
+                if kp is not None:
+                    self.kv_off = self._offsets(kp, Sk, self.Lk, "kv_positions")
+            if fn.alibi_slopes is not None:
+                if fn.alibi_slopes.numel() != self.H:
+                    raise ValueError("alibi slopes must have one entry per head")
+                self.fn = BiasFn(fn.causal, fn.window, fn.segments, fn.prefix,
+                                 fn.alibi_slopes.to(device=dev, dtype=torch.float32).contiguous())
+
+    def _offsets(self, pos, S, L, name):
+        """Positions must be consecutive inside each shard and equal across the batch."""
+        if tuple(pos.shape) != (self.B, S):
+            raise ValueError(f"{name} must have shape {(self.B, S)}, got {tuple(pos.shape)}")
+        pos = pos.to(torch.int64)
+        starts = pos[:, ::L]
+        expect = (starts[:, :, None] + torch.arange(L, device=pos.device)[None, None, :]).reshape(self.B, S)
+        if not torch.equal(expect, pos) or not bool((starts == starts[:1]).all()):
+            raise NotImplementedError(
+                f"{name}: the kernels take one position offset per shard, so positions must be "
+                "consecutive inside every shard and identical across the batch")
+        return [int(x) for x in starts[0].tolist()]
+
+    def block_bias(self, qs: int, ks: int) -> Optional[BlockBias]:
+        """Bias of (query shard qs, key/value shard ks)."""
+        if self.fn is None:
+            return None
+        sl_q = slice(qs * self.Lq, (qs + 1) * self.Lq)
+        sl_k = slice(ks * self.Lk, (ks + 1) * self.Lk)
+        return BlockBias(
+            self.fn, self.q_off[qs], self.kv_off[ks],
+            None if self.q_seg is None else self.q_seg[:, sl_q],
+            None if self.kv_seg is None else self.kv_seg[:, sl_k],
+            None if self.q_pre is None else self.q_pre[:, sl_q],
+            None if self.kv_pre is None else self.kv_pre[:, sl_k])
+
+
+def _shard_bhld(x, s, L):
+    """Shard s of a [b, S, h, d] array, viewed as [b, h, L, d] (no copy)."""
+    return x[:, s * L:(s + 1) * L].permute(0, 2, 1, 3)
+
+
+def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=None):
+    n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
+    dev = q.device
+    out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
+    lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    o, m, l = init_carry(B, H, Lq, D, dev)
+    for r in range(n):
+        if r:
+            reset_carry(o, m, l)
+        qr = _shard_bhld(q, r, Lq)
+        for t in range(n):
+            src = (r - t) % n  # ring.py:51-55: after t rotations device r holds shard r - t
+            fwd_block(qr, _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk), plan.block_bias(r, src),
+                      o, m, l, sm_scale)
+            if carries_out is not None:
+                carries_out.append((r, t, o.clone(), m.clone(), l.clone()))
+        finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
+    return out, lse
+
+
+def _ring_backward(q, k, v, out, lse, do, plan: _RingPlan, sm_scale):
+    n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
+    dev = q.device
+    delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    for s in range(n):
+        precompute_delta(_shard_bhld(out, s, Lq), _shard_bhld(do, s, Lq), delta[s])
+    dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
+    dk_acc = torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)
+    dv_acc = torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    for r in range(n):  # device r keeps its key/value shard and dk/dv (ring.py:183-200)
+        dk_acc.zero_()
+        dv_acc.zero_()
+        kr, vr = _shard_bhld(k, r, Lk), _shard_bhld(v, r, Lk)
+        for t in range(n):
+            src = (r - t) % n  # the query-side shard visiting device r at step t (ring.py:195)
+            _bwd_step(_shard_bhld(q, src, Lq), kr, vr, _shard_bhld(do, src, Lq), lse[src], delta[src],
+                      dq_acc[src], dk_acc, dv_acc, plan.block_bias(src, r), sm_scale)
+        _finalize_grad(dk_acc, _shard_bhld(dk, r, Lk))
+        _finalize_grad(dv_acc, _shard_bhld(dv, r, Lk))
+    for s in range(n):
+        _finalize_grad(dq_acc[s], _shard_bhld(dq, s, Lq))
+    return dq, dk, dv
+
+
+class _RingAttentionFn(torch.autograd.Function):
+    """custom_vjp of the reference (ring.py:214-243): forward saves (q, k, v, o, L)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, plan, sm_scale, out_dtype):
+        out, lse = _ring_forward(q, k, v, plan, sm_scale, out_dtype)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.plan, ctx.sm_scale = plan, sm_scale
+        ctx.mark_non_differentiable(lse)
+        return out, lse
+
+    @staticmethod
+    def backward(ctx, do, _dlse):
+        q, k, v, out, lse = ctx.saved_tensors
+        do = _kernel_ready(do)
+        dq, dk, dv = _ring_backward(q, k, v, out, lse, do, ctx.plan, ctx.sm_scale)
+        return dq, dk, dv, None, None, None
+
+
+def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Optional[BiasFn] = None, bias_q_kwargs=None,
+                            bias_kv_kwargs=None, sm_scale: Optional[float] = None,
+                            block_impl: str = "hip", out_dtype=None):
+    """``ring_attention`` that also returns the logsumexp ``[b, h, S]`` (the ``L`` residual of
+    ring.py:135)."""
+    if block_impl not in _IMPLS:
+        raise ValueError(block_impl)
+    if bias_fn is not None and not isinstance(bias_fn, BiasFn):
+        raise TypeError("bias_fn must be a ring_attention.BiasFn: arbitrary Python callables "
+                        "cannot be evaluated inside the kernels")
+    _require_gpu(q)
+    _lib.load()
+    n = _axis_size(axis_name)
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be [b, l, h, d]")
+    d_true = q.shape[-1]
+    if k.shape[-1] != d_true or v.shape[-1] != d_true:
+        raise ValueError("q, k and v must share the head dim")
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(d_true)  # ring.py:287-288
+    in_dtype = q.dtype
+    if out_dtype is None:
+        out_dtype = torch.float32 if in_dtype == torch.float32 else torch.bfloat16
+    d_pad = 64 if d_true <= 64 else 128
+    if d_true > 128:
+        raise ValueError("head dims above 128 are not supported")
+    if d_pad != d_true:
+        pad = (0, d_pad - d_true)
+        q, k, v = (torch.nn.functional.pad(x, pad) for x in (q, k, v))
+    q, k, v = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
+    plan = _RingPlan(q, k, n, bias_fn, bias_q_kwargs, bias_kv_kwargs)
+    out, lse = _RingAttentionFn.apply(q, k, v, plan, float(sm_scale), out_dtype)
+    if d_pad != d_true:
+        out = out[..., :d_true]
+    if in_dtype not in (torch.float32, torch.bfloat16):
+        out = out.to(in_dtype)
+    lse_full = lse.permute(1, 2, 0, 3).reshape(plan.B, plan.H, n * plan.Lq)
+    return out, lse_full
+
+
+def ring_attention(q, k, v, axis_name, bias_fn: Optional[BiasFn] = None, bias_q_kwargs=None,
+                   bias_kv_kwargs=None, sm_scale: Optional[float] = None, block_impl: str = "hip"):
+    """Ring attention - general (reference ``ring_attention``, ring.py:246-325).
+
+    Args:
+        q, k, v: ``[b, S, h, d]`` global arrays on the GPU (see the module docstring).
+        axis_name: ``RingAxis`` / int ring size: how many shards the sequence is cut into.
+        bias_fn: optional ``BiasFn`` describing the block-wise attention bias.
+        bias_q_kwargs / bias_kv_kwargs: query- / key-aligned ``[b, S]`` arrays the bias needs
+            (``q_segment_ids``, ``q_positions``, ``q_prefix_mask`` and their ``kv_`` twins).
+        sm_scale: softmax scale, 1/sqrt(d) if unspecified.
+        block_impl: ``"hip"`` (``"pallas"`` is accepted as an alias); anything else raises
+            ``ValueError`` as the reference does (ring.py:312).
+    Returns:
+        attention output ``[b, S, h, d]``; differentiable w.r.t. q, k, v.
+    """
+    out, _ = ring_attention_with_lse(q, k, v, axis_name, bias_fn, bias_q_kwargs, bias_kv_kwargs,
+                                     sm_scale, block_impl)
+    return out
+
+
+def ring_self_attention(q, k, v, mesh, pspec=None, sm_scale: Optional[float] = None,
+                        causal: bool = False, segment_ids=None, positions=None, prefix_mask=None,
+                        block_impl: str = "hip"):
+    """Ring attention for self-attention (reference ``ring_self_attention``, ring.py:328-449).
+
+    Supports full bidirectional attention (default), block-sparse attention via
+    ``segment_ids``, causal attention (requires ``positions``) and prefix-LM attention via
+    ``prefix_mask`` (requires ``positions``), and their combinations.  ``mesh`` gives the
+    ring size (``RingAxis`` or int); ``pspec`` is accepted for signature compatibility."""
+    if causal:
+        assert positions is not None, "positions are requried for causal attention"
+        assert prefix_mask is None, "causal attention does not support prefix_mask"
+    if prefix_mask is not None:
+        assert positions is not None, "positions are requried for prefixlm attention"
+        assert not causal
+    fn = BiasFn(causal=causal, segments=segment_ids is not None, prefix=prefix_mask is not None)
+    has_bias = causal or segment_ids is not None or prefix_mask is not None
+    q_kw = {"q_segment_ids": segment_ids, "q_positions": positions, "q_prefix_mask": prefix_mask}
+    kv_kw = {"kv_segment_ids": segment_ids, "kv_positions": positions, "kv_prefix_mask": prefix_mask}
+    return ring_attention(q, k, v, mesh, bias_fn=fn if has_bias else None,
+                          bias_q_kwargs=q_kw if has_bias else None,
+                          bias_kv_kwargs=kv_kw if has_bias else None, sm_scale=sm_scale,
+                          block_impl=block_impl)
