@@ -141,6 +141,12 @@ int ra_bwd_delta(const void* out, int32_t out_dtype, int64_t out_stride_b,
  * (ring.py:140-157) and the accumulation ring.py:191-193. */
 int ra_bwd_step(const ra_bwd_step_params* p, void* stream);
 
+/* ra_bwd_step restricted to a subset of its kernels: parts is a bit mask, 1 = the dK/dV
+ * kernel (the q-loop of ring_kernel.py:343-367), 2 = the dQ kernel (the dq product that the
+ * reference adds atomically, ring_kernel.py:369-374).  parts = 3 is ra_bwd_step.  Lets a
+ * caller time or schedule the two halves separately. */
+int ra_bwd_step_parts(const ra_bwd_step_params* p, int32_t parts, void* stream);
+
 /* Cast an fp32 accumulator [B,H,L,D] to a strided bf16 tensor (the final dq/dk/dv in the
  * caller's layout).   Replaces the output transposes ring.py:208-210. */
 int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t out_stride_h,

@@ -166,7 +166,8 @@ def mha_dense(q, k, v, bias=None, sm_scale=None, dtype=np.float64):
                 p = np.exp(s - m)
                 l = p.sum(axis=-1, keepdims=True)
                 out[b, :, h] = (p @ v[b, :, h]) / l
-                lse[b, h] = (m + np.log(l))[:, 0]
+                # a row with no visible key: m = -inf, and ring.py:135 yields -inf + log(0) = -inf
+                lse[b, h] = np.where(np.isneginf(m), NEG_INF, m + np.log(l))[:, 0]
     return out, lse
 
 
@@ -201,7 +202,7 @@ def fwd_block(q, k, v, bias, o, m_prev, l, sm_scale):
     """One ring step of the online softmax, restating ring.py:58-76.
     q [b h lq d], k/v [b h lk d], bias [b h|1 lq lk] or None, o [b h lq d], m_prev/l
     [b h lq].  Returns the unnormalised (o, m, l)."""
-    s = np.einsum("bhqd,bhkd->bhqk", q, k) * sm_scale
+    s = np.matmul(q, np.swapaxes(k, -1, -2)) * sm_scale
     if bias is not None:
         s = s + bias
     m = np.maximum(m_prev, s.max(axis=-1))
@@ -210,7 +211,7 @@ def fwd_block(q, k, v, bias, o, m_prev, l, sm_scale):
         correction = np.where(np.isneginf(m) & np.isneginf(m_prev), 0.0, correction)
         p = np.exp(s - m[..., None])
         p = np.where(np.isneginf(m)[..., None], 0.0, p)
-    pv = np.einsum("bhqk,bhkd->bhqd", p, v)
+    pv = np.matmul(p, v)
     o = o * correction[..., None] + pv
     l = correction * l + p.sum(axis=-1)
     return o, m, l
@@ -218,17 +219,17 @@ def fwd_block(q, k, v, bias, o, m_prev, l, sm_scale):
 
 def bwd_block(q, k, v, bias, o, L, do, sm_scale):
     """One ring step of the backward pass, restating ring.py:140-157."""
-    s = np.einsum("bhqd,bhkd->bhqk", q, k) * sm_scale
+    s = np.matmul(q, np.swapaxes(k, -1, -2)) * sm_scale
     if bias is not None:
         s = s + bias
     with np.errstate(invalid="ignore"):
         p = np.exp(s - L[..., None])
-    dv = np.einsum("bhqk,bhqd->bhkd", p, do)
-    dp = np.einsum("bhqd,bhkd->bhqk", do, v)
+    dv = np.matmul(np.swapaxes(p, -1, -2), do)
+    dp = np.matmul(do, np.swapaxes(v, -1, -2))
     delta = np.sum(do * o, axis=-1, keepdims=True)
     ds = p * (dp - delta) * sm_scale
-    dq = np.einsum("bhqk,bhkd->bhqd", ds, k)
-    dk = np.einsum("bhqk,bhqd->bhkd", ds, q)
+    dq = np.matmul(ds, k)
+    dk = np.matmul(np.swapaxes(ds, -1, -2), q)
     return dq, dk, dv
 
 

@@ -208,9 +208,12 @@ int ra_bwd_delta(const void* out, int32_t out_dtype, int64_t out_stride_b, int64
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_delta launch");
 }
 
-int ra_bwd_step(const ra_bwd_step_params* p, void* stream) {
+int ra_bwd_step(const ra_bwd_step_params* p, void* stream) { return ra_bwd_step_parts(p, 3, stream); }
+
+int ra_bwd_step_parts(const ra_bwd_step_params* p, int32_t parts, void* stream) {
   int rc = ra_bwd_step_check(p);
   if (rc) return rc;
+  if (parts < 1 || parts > 3) return fail(RA_ERR_SHAPE, "parts must be 1, 2 or 3 (got %d)", parts);
   if (ra_step_is_skippable(&p->bias, p->Lq, p->Lk)) return RA_OK;  // contributes nothing
   ra::BwdArgs a;
   a.q = to_arg(p->q);
@@ -229,7 +232,7 @@ int ra_bwd_step(const ra_bwd_step_params* p, void* stream) {
   a.scale2 = p->sm_scale * kLog2eHost;
   a.sm_scale = p->sm_scale;
   a.bias = to_bias(p->bias);
-  hipError_t e = ra::launch_bwd_step(a, p->D, is_general(p->bias.flags), (hipStream_t)stream);
+  hipError_t e = ra::launch_bwd_step(a, p->D, is_general(p->bias.flags), parts, (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_step launch");
 }
 

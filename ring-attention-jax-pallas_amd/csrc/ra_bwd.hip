@@ -587,8 +587,8 @@ hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long lon
 
 constexpr int kNkb = 1;  // 32-key blocks per wave in dkdv_kernel
 
-hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, hipStream_t stream) {
-  {
+hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, int parts, hipStream_t stream) {
+  if (parts & 1) {
     const int keys_wg = 4 * 32 * kNkb;
     const int nkt = (a.Lk + keys_wg - 1) / keys_wg;
     dim3 grid((unsigned)(a.B * a.H * nkt)), block(256);
@@ -602,7 +602,7 @@ hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, hipStream_t st
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
   }
-  {
+  if (parts & 2) {
     const int nqt = (a.Lq + kDqRows - 1) / kDqRows;
     dim3 grid((unsigned)(a.B * a.H * nqt)), block(kDqThreads);
     if (D == 128) {

@@ -67,6 +67,7 @@ EXPORTS = {
                                C.POINTER(RaTensor), C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
                                C.c_int32, C.c_void_p]),
     "ra_bwd_step": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_void_p]),
+    "ra_bwd_step_parts": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
     "ra_bwd_finalize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32,
                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "ra_step_is_skippable": (C.c_int, [C.POINTER(RaBias), C.c_int32, C.c_int32]),

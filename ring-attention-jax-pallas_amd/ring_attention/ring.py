@@ -152,7 +152,7 @@ def precompute_delta(out, do, delta=None):
     return delta
 
 
-def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale):
+def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, parts=3):
     lib = _lib.load()
     B, H, Lq, D = q.shape
     p = _lib.RaBwdStepParams()
@@ -162,7 +162,7 @@ def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale):
     p.lse, p.delta = lse.data_ptr(), delta.data_ptr()
     p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     p.bias = _bias_struct(bias, q.device)
-    _lib.check("ra_bwd_step", lib.ra_bwd_step(C.byref(p), _stream()))
+    _lib.check("ra_bwd_step", lib.ra_bwd_step_parts(C.byref(p), parts, _stream()))
 
 
 def bwd_block(q, k, v, bias: Optional[BlockBias], o, L, do, sm_scale: float):
@@ -278,7 +278,28 @@ def _shard_bhld(x, s, L):
     return x[:, s * L:(s + 1) * L].permute(0, 2, 1, 3)
 
 
-def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=None):
+class _NoTimer:
+    """Default launch observer: does nothing.  A benchmark passes an object whose
+    ``span(kind, qs, ks)`` context manager brackets one kernel launch with stream events."""
+
+    class _Span:
+        def __enter__(self):
+            return self
+
+        def __exit__(self, *exc):
+            return False
+
+    _span = _Span()
+    split_bwd = False
+
+    def span(self, kind, qs, ks):
+        return self._span
+
+
+_NO_TIMER = _NoTimer()
+
+
+def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=None, timer=_NO_TIMER):
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
@@ -290,15 +311,16 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
         qr = _shard_bhld(q, r, Lq)
         for t in range(n):
             src = (r - t) % n  # ring.py:51-55: after t rotations device r holds shard r - t
-            fwd_block(qr, _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk), plan.block_bias(r, src),
-                      o, m, l, sm_scale)
+            with timer.span("fwd", r, src):
+                fwd_block(qr, _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk),
+                          plan.block_bias(r, src), o, m, l, sm_scale)
             if carries_out is not None:
                 carries_out.append((r, t, o.clone(), m.clone(), l.clone()))
         finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
     return out, lse
 
 
-def _ring_backward(q, k, v, out, lse, do, plan: _RingPlan, sm_scale):
+def _ring_backward(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
@@ -314,8 +336,15 @@ def _ring_backward(q, k, v, out, lse, do, plan: _RingPlan, sm_scale):
         kr, vr = _shard_bhld(k, r, Lk), _shard_bhld(v, r, Lk)
         for t in range(n):
             src = (r - t) % n  # the query-side shard visiting device r at step t (ring.py:195)
-            _bwd_step(_shard_bhld(q, src, Lq), kr, vr, _shard_bhld(do, src, Lq), lse[src], delta[src],
-                      dq_acc[src], dk_acc, dv_acc, plan.block_bias(src, r), sm_scale)
+            args = (_shard_bhld(q, src, Lq), kr, vr, _shard_bhld(do, src, Lq), lse[src], delta[src],
+                    dq_acc[src], dk_acc, dv_acc, plan.block_bias(src, r), sm_scale)
+            if timer.split_bwd:
+                with timer.span("bwd_dkdv", src, r):
+                    _bwd_step(*args, parts=1)
+                with timer.span("bwd_dq", src, r):
+                    _bwd_step(*args, parts=2)
+            else:
+                _bwd_step(*args)
         _finalize_grad(dk_acc, _shard_bhld(dk, r, Lk))
         _finalize_grad(dv_acc, _shard_bhld(dv, r, Lk))
     for s in range(n):

@@ -1,0 +1,122 @@
+"""CPU-only checks of the C ABI: the library loads, exports what include/ring_attention_hip.h
+declares, rejects bad arguments before touching a GPU, and classifies skippable ring steps
+exactly like a brute-force evaluation of the bias."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oracle import ring_oracle as R
+from ring_attention import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "ring_attention_hip.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ra_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = _declared()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    assert sorted(_lib.EXPORTS) == names, "python binding table and header disagree"
+    assert lib.ra_version() >= 1000
+
+
+def test_struct_layout_matches_header():
+    # sizes implied by the header with natural alignment on x86-64
+    assert C.sizeof(_lib.RaTensor) == 32
+    assert C.sizeof(_lib.RaBias) == 8 + 16 + 16 + 16 + 16 + 16 + 8
+    assert C.sizeof(_lib.RaFwdStepParams) == 24 + 3 * 32 + 24 + C.sizeof(_lib.RaBias)
+    assert C.sizeof(_lib.RaBwdStepParams) == 24 + 4 * 32 + 40 + C.sizeof(_lib.RaBias)
+
+
+def _good_fwd():
+    p = _lib.RaFwdStepParams()
+    p.B, p.H, p.Lq, p.Lk, p.D = 1, 2, 64, 64, 128
+    p.sm_scale = 0.1
+    for t in (p.q, p.k, p.v):
+        t.ptr, t.stride_b, t.stride_h, t.stride_l = 0x1000, 64 * 256, 128, 256
+    p.o = p.m = p.l = 0x2000
+    return p
+
+
+def _good_bwd():
+    p = _lib.RaBwdStepParams()
+    p.B, p.H, p.Lq, p.Lk, p.D = 1, 2, 64, 64, 64
+    p.sm_scale = 0.1
+    for t in (p.q, p.k, p.v, p.dout):
+        t.ptr, t.stride_b, t.stride_h, t.stride_l = 0x1000, 64 * 128, 64, 128
+    p.lse = p.delta = p.dq = p.dk = p.dv = 0x2000
+    return p
+
+
+def test_check_accepts_good_params(lib):
+    assert lib.ra_fwd_step_check(C.byref(_good_fwd())) == 0
+    assert lib.ra_bwd_step_check(C.byref(_good_bwd())) == 0
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda p: setattr(p, "D", 96), -3),
+    (lambda p: setattr(p, "D", 256), -3),
+    (lambda p: setattr(p, "Lq", 0), -2),
+    (lambda p: setattr(p, "B", -1), -2),
+    (lambda p: setattr(p.q, "ptr", None), -1),
+    (lambda p: setattr(p.k, "ptr", 0x1008), -4),
+    (lambda p: setattr(p.v, "stride_l", 129), -4),
+    (lambda p: setattr(p, "o", None), -1),
+    (lambda p: setattr(p, "sm_scale", float("nan")), -2),
+    (lambda p: setattr(p.bias, "flags", 64), -5),
+    (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_WINDOW), -5),            # window == 0
+    (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL | _lib.RA_BIAS_PREFIX), -5),
+    (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_SEGMENT), -1),           # no id arrays
+    (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_ALIBI), -1),             # no slopes
+    (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL), setattr(p.bias, "q_offset", -5)), -5),
+])
+def test_fwd_step_rejects_bad_params_without_a_gpu(lib, mutate, code):
+    p = _good_fwd()
+    mutate(p)
+    assert lib.ra_fwd_step_check(C.byref(p)) == code
+    assert lib.ra_fwd_step(C.byref(p), None) == code  # validation comes before any HIP call
+    assert lib.ra_last_error() != b""
+
+
+def test_bwd_step_rejects_bad_params_without_a_gpu(lib):
+    p = _good_bwd()
+    p.dk = None
+    assert lib.ra_bwd_step(C.byref(p), None) == -1
+    p = _good_bwd()
+    p.dout.stride_h = 3
+    assert lib.ra_bwd_step(C.byref(p), None) == -4
+    p = _good_bwd()
+    assert lib.ra_bwd_step_parts(C.byref(p), 7, None) == -2
+    assert lib.ra_fwd_step(None, None) == -1
+    assert lib.ra_fwd_init(None, None, None, 1, 1, 1, 64, None) == -1
+    assert lib.ra_fwd_finalize(0x10, 0x10, 0x10, 0x10, 5, 8, 8, 8, 0x10, 1, 1, 1, 64, None) == -7
+
+
+@pytest.mark.parametrize("flags,window", [(1, 0), (3, 7), (2, 7), (3, 64), (2, 1), (0, 0), (8, 0)])
+def test_step_is_skippable_matches_brute_force(lib, flags, window):
+    Lq, Lk = 16, 24
+    for q_off in (0, 16, 40, 100):
+        for kv_off in (0, 24, 48, 96):
+            b = _lib.RaBias()
+            b.flags, b.window, b.q_offset, b.kv_offset = flags, window, q_off, kv_off
+            got = lib.ra_step_is_skippable(C.byref(b), Lq, Lk)
+            qp = (q_off + np.arange(Lq))[None]
+            kp = (kv_off + np.arange(Lk))[None]
+            fn = R.make_bias_fn(causal=bool(flags & 1), window=window if flags & 2 else None,
+                                use_prefix=bool(flags & 8))
+            pm_q = np.ones((1, Lq), dtype=np.int32); pm_k = np.ones((1, Lk), dtype=np.int32)
+            bias = fn(q_positions=qp, kv_positions=kp, q_prefix_mask=pm_q, kv_prefix_mask=pm_k)
+            want = int(np.all(np.isneginf(bias)))
+            if flags & 8:
+                want = 0  # prefix masks are data dependent: never skipped on the host
+            assert got == want, (flags, window, q_off, kv_off)

@@ -1,0 +1,369 @@
+"""GPU parity tests: the HIP kernels (through the C ABI) against the CPU oracle on the same
+seeded inputs.  Tolerances are BASELINE's: forward output max-abs error <= 1e-2 and
+logsumexp <= 1e-3 for bf16 inputs against the fp64 oracle on the same bf16-rounded values,
+dq/dk/dv relative error <= 2e-2 (max|diff| / max|ref| and Frobenius)."""
+import glob
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import ring_attention as ra
+from oracle import ring_oracle as R
+from ring_attention import ring as rr
+
+pytestmark = pytest.mark.gpu
+
+OUT_TOL, LSE_TOL, GRAD_TOL = 1e-2, 1e-3, 2e-2
+
+
+def _dev(x, device, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(x)).to(device)
+    return t.to(dtype) if dtype is not None else t
+
+
+def _rel(a, b):
+    """max|diff| / max|ref| and the Frobenius ratio.  The denominators are floored at 0.05 (per
+    element) so that a gradient that is exactly zero in real arithmetic (a window of one key:
+    dq = dk = 0) is judged on its absolute size instead of on rounding noise."""
+    return (np.abs(a - b).max() / max(np.abs(b).max(), 0.05),
+            np.linalg.norm(a - b) / max(np.linalg.norm(b), 0.05 * np.sqrt(b.size)))
+
+
+def _run_hip(device, q, k, v, do, n, fn, qkw, kvkw, sm_scale=None):
+    tq, tk, tv = (_dev(x, device, torch.bfloat16).requires_grad_(True) for x in (q, k, v))
+    tqkw = {a: _dev(b, device) for a, b in (qkw or {}).items()} or None
+    tkvkw = {a: _dev(b, device) for a, b in (kvkw or {}).items()} or None
+    out, lse = ra.ring_attention_with_lse(tq, tk, tv, n, bias_fn=fn, bias_q_kwargs=tqkw,
+                                          bias_kv_kwargs=tkvkw, sm_scale=sm_scale, out_dtype=torch.float32)
+    grads = None
+    if do is not None:
+        out.backward(_dev(do, device, torch.float32))
+        grads = tuple(t.grad.float().cpu().numpy() for t in (tq, tk, tv))
+    torch.cuda.synchronize()
+    return out.detach().cpu().numpy(), lse.cpu().numpy(), grads
+
+
+def _check(device, name, B, Sq, Sk, H, D, n, fn=None, ofn=None, qkw=None, kvkw=None, std=1.0, seed=0,
+           grads=True):
+    print(f"[parity] {name}: B={B} Sq={Sq} Sk={Sk} H={H} D={D} ring={n} seed={seed}", flush=True)
+    q, k, v, do = R.make_inputs(seed, B, Sq, Sk, H, D, std=std)
+    out, lse, g = _run_hip(device, q, k, v, do if grads else None, n, fn, qkw, kvkw)
+    oq, okv = dict(qkw or {}), dict(kvkw or {})
+    bias = None
+    if ofn is not None:
+        oq.setdefault("q_positions", np.broadcast_to(np.arange(Sq), (B, Sq)))
+        okv.setdefault("kv_positions", np.broadcast_to(np.arange(Sk), (B, Sk)))
+        bias = ofn(**oq, **okv)
+    want, want_lse = R.mha_dense(q, k, v, bias)
+    np.testing.assert_array_equal(np.isnan(out), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.abs(out - want)[ok].max() <= OUT_TOL
+    okl = np.isfinite(want_lse)
+    np.testing.assert_array_equal(np.isneginf(lse), np.isneginf(want_lse))
+    assert np.abs(lse[okl] - want_lse[okl]).max() <= LSE_TOL
+    if grads and ok.all():
+        for got, ref, nm in zip(g, R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
+            mx, fro = _rel(got, ref)
+            assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+
+
+# ---- the reference's own test shapes (ring_test.py:48-53, :104-111), 8 shards, B=2 -------------
+@pytest.mark.parametrize("seed,q_len,kv_len,h,d", [
+    (0, 24, 16, 1, 2), (1, 128, 64, 4, 64), (2, 64, 512, 4, 16), (3, 128, 2048, 2, 128),
+    (3, 2048, 128, 2, 128), (3, 2048, 2048, 4, 128)])
+def test_reference_shapes_no_bias(device, seed, q_len, kv_len, h, d):
+    _check(device, "ref-shape", 2, q_len, kv_len, h, d, 8, seed=seed)
+
+
+@pytest.mark.parametrize("seed,q_len,kv_len,h,d", [
+    (0, 24, 16, 1, 2), (1, 128, 64, 4, 64), (2, 64, 512, 4, 16), (3, 2048, 2048, 4, 128)])
+def test_reference_shapes_segment_bias(device, seed, q_len, kv_len, h, d):
+    # ring_test.py:174-300: random ids in [0, q_len // 5): rows without a matching key give NaN
+    rng = np.random.default_rng(seed)
+    qs = rng.integers(0, q_len // 5, (2, q_len)).astype(np.int32)
+    ks = rng.integers(0, q_len // 5, (2, kv_len)).astype(np.int32)
+    _check(device, "ref-shape-segments", 2, q_len, kv_len, h, d, 8, ra.segment_bias(),
+           R.make_bias_fn(use_segments=True), {"q_segment_ids": qs}, {"kv_segment_ids": ks}, seed=seed)
+
+
+@pytest.mark.parametrize("seed,length,h,d", [(0, 16, 1, 2), (1, 128, 4, 64), (2, 512, 4, 16), (4, 2048, 4, 64)])
+def test_reference_shapes_self_attention(device, seed, length, h, d):
+    # ring_test.py:320-378: ring_self_attention, causal + segments in [0, 5), positions = arange
+    print(f"[parity] self-attention length={length} h={h} d={d}", flush=True)
+    q, k, v, _ = R.make_inputs(seed, 2, length, length, h, d)
+    seg = np.random.default_rng(seed).integers(0, 5, (2, length)).astype(np.int32)
+    pos = np.broadcast_to(np.arange(length), (2, length)).copy()
+    out = ra.ring_self_attention(_dev(q, device), _dev(k, device), _dev(v, device), ra.RingAxis("sp", 8), None,
+                                 causal=True, segment_ids=_dev(seg, device), positions=_dev(pos, device))
+    assert out.dtype == torch.float32 and out.shape == q.shape
+    bias = R.make_bias_fn(causal=True, use_segments=True)(
+        q_segment_ids=seg, kv_segment_ids=seg, q_positions=pos, kv_positions=pos)
+    want, _ = R.mha_dense(q, k, v, bias)
+    assert np.abs(out.cpu().numpy() - want).max() <= OUT_TOL
+
+
+# ---- bias functors --------------------------------------------------------------------------------
+def test_causal_c1_config(device):
+    # BASELINE config 1: B=1 H=4 S=1024 D=64, ring of 4 shards of 256, causal
+    _check(device, "C1", 1, 1024, 1024, 4, 64, 4, ra.causal_bias(), R.make_bias_fn(causal=True))
+
+
+def test_ragged_lengths(device):
+    _check(device, "ragged", 1, 200, 136, 2, 128, 1)
+    _check(device, "ragged-causal", 2, 3 * 37, 3 * 37, 2, 64, 3, ra.causal_bias(), R.make_bias_fn(causal=True))
+
+
+def test_causal_d128_ring8(device):
+    _check(device, "causal-d128", 2, 2048, 2048, 4, 128, 8, ra.causal_bias(), R.make_bias_fn(causal=True))
+
+
+@pytest.mark.parametrize("window,causal", [(300, True), (64, True), (1, True), (200, False)])
+def test_sliding_window(device, window, causal):
+    _check(device, f"window{window}", 1, 2048, 2048, 2, 128, 8, ra.sliding_window_bias(window, causal),
+           R.make_bias_fn(causal=causal, window=window), std=0.5)
+
+
+def test_sorted_segments_and_alibi(device):
+    seg = R.geometric_segment_ids(0, 2, 2048, 300)
+    _check(device, "segments-sorted", 2, 2048, 2048, 2, 128, 4, ra.segment_bias(),
+           R.make_bias_fn(use_segments=True), {"q_segment_ids": seg}, {"kv_segment_ids": seg})
+    sl = R.alibi_slopes(4)
+    _check(device, "segments+alibi", 1, 2048, 2048, 4, 128, 4, ra.segment_bias() + ra.alibi_bias(sl),
+           R.make_bias_fn(use_segments=True, alibi=sl), {"q_segment_ids": seg[:1]}, {"kv_segment_ids": seg[:1]})
+    _check(device, "causal+alibi", 1, 1024, 1024, 4, 64, 4, ra.causal_bias() + ra.alibi_bias(sl),
+           R.make_bias_fn(causal=True, alibi=sl))
+
+
+def test_prefix_lm(device):
+    pm = (np.arange(512)[None, :] < np.array([[100], [300]])).astype(np.int32)
+    _check(device, "prefix", 2, 512, 512, 2, 64, 4, ra.prefix_lm_bias(), R.make_bias_fn(use_prefix=True),
+           {"q_prefix_mask": pm}, {"kv_prefix_mask": pm})
+    seg = np.sort(np.random.default_rng(3).integers(0, 3, (2, 512)), axis=1).astype(np.int32)
+    _check(device, "prefix+segments", 2, 512, 512, 2, 128, 4, ra.prefix_lm_bias() + ra.segment_bias(),
+           R.make_bias_fn(use_prefix=True, use_segments=True),
+           {"q_prefix_mask": pm, "q_segment_ids": seg}, {"kv_prefix_mask": pm, "kv_segment_ids": seg})
+
+
+def test_shard_positions_with_offsets(device):
+    # positions restart from an arbitrary offset in every shard
+    B, S, n = 1, 512, 4
+    starts = np.array([1000, 0, 5000, 128])
+    pos = (starts[:, None] + np.arange(S // n)[None, :]).reshape(1, S)
+    _check(device, "offsets", B, S, S, 2, 64, n, ra.causal_bias(), R.make_bias_fn(causal=True),
+           {"q_positions": pos}, {"kv_positions": pos})
+
+
+# ---- golden fixtures ----------------------------------------------------------------------------------
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz"))))
+def test_golden_fixtures(device, path):
+    z = np.load(path)
+    name = os.path.basename(path)
+    print(f"[parity] golden {name}", flush=True)
+    fn, qkw, kvkw = None, None, None
+    if "causal_segments" in name:
+        fn = ra.causal_bias() + ra.segment_bias()
+        qkw, kvkw = {"q_segment_ids": z["seg"]}, {"kv_segment_ids": z["seg"]}
+    elif "causal" in name:
+        fn = ra.causal_bias()
+    elif "window_alibi" in name:
+        fn = ra.sliding_window_bias(40) + ra.alibi_bias(z["slopes"])
+    out, lse, g = _run_hip(device, z["q"], z["k"], z["v"], z["do"], int(z["ring"]), fn, qkw, kvkw)
+    assert np.abs(out - z["out"]).max() <= OUT_TOL
+    assert np.abs(lse - z["lse"]).max() <= LSE_TOL
+    for got, key in zip(g, ("dq", "dk", "dv")):
+        mx, fro = _rel(got, z[key])
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL, (key, mx, fro)
+
+
+# ---- per-step carry semantics ----------------------------------------------------------------------------
+def test_per_step_carries_match_oracle(device):
+    """(o, m, l) after every ring step equals the oracle's blockwise carry (ring.py:104-132)."""
+    B, S, H, D, n = 1, 1024, 2, 64, 4
+    q, k, v, _ = R.make_inputs(21, B, S, S, H, D)
+    pos = np.broadcast_to(np.arange(S), (B, S))
+    _, _, want = R.ring_attention(q, k, v, n, R.make_bias_fn(causal=True), {"q_positions": pos},
+                                  {"kv_positions": pos}, return_carries=True)
+    tq, tk, tv = (_dev(x, device, torch.bfloat16) for x in (q, k, v))
+    plan = rr._RingPlan(tq, tk, n, ra.causal_bias(), None, None)
+    got = []
+    rr._ring_forward(tq, tk, tv, plan, 1 / math.sqrt(D), torch.float32, carries_out=got)
+    torch.cuda.synchronize()
+    for r, t, o, m, l in got:
+        wo, wm, wl = want[r][t]
+        m_, l_, o_ = m.cpu().numpy(), l.cpu().numpy(), o.cpu().numpy()
+        np.testing.assert_array_equal(np.isneginf(m_), np.isneginf(wm))
+        fin = np.isfinite(wm)
+        assert np.abs(m_ - wm)[fin].max() <= 1e-4
+        np.testing.assert_allclose(l_, wl, rtol=5e-3, atol=1e-6)
+        assert np.abs(o_ - wo).max() <= 1e-2 * max(1.0, np.abs(wo).max())
+
+
+def test_block_api_matches_reference_contract(device):
+    """fwd_block / bwd_block on [b, h, l, d] tensors (ring_kernel.py:123-131, :202-211)."""
+    B, H, Lq, Lk, D = 2, 2, 256, 128, 128
+    q, k, v, do = R.make_inputs(5, B, Lq, Lk, H, D)
+    hq, hk, hv, hdo = (np.ascontiguousarray(np.transpose(x, (0, 2, 1, 3))) for x in (q, k, v, do))
+    tq, tk, tv, tdo = (_dev(x, device, torch.bfloat16) for x in (hq, hk, hv, hdo))
+    o, m, l = rr.init_carry(B, H, Lq, D, device)
+    assert torch.all(o == 0) and torch.all(l == 0) and torch.all(torch.isneginf(m))
+    scale = 1 / math.sqrt(D)
+    o, m, l = ra.fwd_block(tq, tk, tv, None, o, m, l, scale)
+    wo, wm, wl = R.fwd_block(hq.astype(np.float64), hk.astype(np.float64), hv.astype(np.float64), None,
+                             np.zeros((B, H, Lq, D)), np.full((B, H, Lq), -np.inf), np.zeros((B, H, Lq)), scale)
+    assert np.abs(m.cpu().numpy() - wm).max() <= 1e-4
+    np.testing.assert_allclose(l.cpu().numpy(), wl, rtol=5e-3)
+    out = (o / l[..., None])
+    L = m + torch.log(l)
+    dq, dk, dv = ra.bwd_block(tq, tk, tv, None, out, L, tdo, scale)
+    wdq, wdk, wdv = R.bwd_block(hq.astype(np.float64), hk.astype(np.float64), hv.astype(np.float64), None,
+                                wo / wl[..., None], wm + np.log(wl), hdo.astype(np.float64), scale)
+    for got, ref in ((dq, wdq), (dk, wdk), (dv, wdv)):
+        mx, fro = _rel(got.cpu().numpy(), ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL
+
+
+def test_delta_kernel(device):
+    B, H, L, D = 2, 3, 100, 64
+    rng = np.random.default_rng(0)
+    out = R.bf16_round(rng.standard_normal((B, L, H, D)).astype(np.float32))
+    do = R.bf16_round(rng.standard_normal((B, L, H, D)).astype(np.float32))
+    want = R.precompute_delta(out, do)
+    for dt in (torch.bfloat16, torch.float32):
+        got = ra.precompute_delta(_dev(out, device, dt).permute(0, 2, 1, 3), _dev(do, device, torch.bfloat16).permute(0, 2, 1, 3))
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+
+
+def test_deterministic_and_layout_independent(device):
+    """No atomics: two runs agree bit for bit; [b,l,h,d] and [b,h,l,d] storage give the same bits."""
+    B, S, H, D, n = 1, 1024, 4, 128, 4
+    q, k, v, do = R.make_inputs(8, B, S, S, H, D)
+    a = _run_hip(device, q, k, v, do, n, ra.causal_bias(), None, None)
+    b = _run_hip(device, q, k, v, do, n, ra.causal_bias(), None, None)
+    np.testing.assert_array_equal(a[0], b[0])
+    for x, y in zip(a[2], b[2]):
+        np.testing.assert_array_equal(x, y)
+    # head-major storage viewed as [b, l, h, d]
+    tq, tk, tv = (_dev(np.ascontiguousarray(np.transpose(x, (0, 2, 1, 3))), device, torch.bfloat16).permute(0, 2, 1, 3)
+                  for x in (q, k, v))
+    assert not tq.is_contiguous()
+    out = ra.ring_attention(tq, tk, tv, n, bias_fn=ra.causal_bias())
+    out_ref = ra.ring_attention(_dev(q, device, torch.bfloat16), _dev(k, device, torch.bfloat16),
+                                _dev(v, device, torch.bfloat16), n, bias_fn=ra.causal_bias())
+    assert torch.equal(out, out_ref)
+
+
+def test_fp32_and_fp16_inputs_are_cast(device):
+    q, k, v, _ = R.make_inputs(2, 1, 256, 256, 2, 64)
+    want, _ = R.mha_dense(q, k, v)
+    out = ra.ring_attention(_dev(q, device), _dev(k, device), _dev(v, device), 2)
+    assert out.dtype == torch.float32 and np.abs(out.cpu().numpy() - want).max() <= OUT_TOL
+    out16 = ra.ring_attention(_dev(q, device, torch.float16), _dev(k, device, torch.float16), _dev(v, device, torch.float16), 2)
+    assert out16.dtype == torch.float16
+    out_bf = ra.ring_attention(_dev(q, device, torch.bfloat16), _dev(k, device, torch.bfloat16), _dev(v, device, torch.bfloat16), 2)
+    assert out_bf.dtype == torch.bfloat16
+    assert np.abs(out_bf.float().cpu().numpy() - want).max() <= 2e-2  # bf16 output rounding on top
+
+
+# ---- BASELINE configs at full size -------------------------------------------------------------------------
+def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, bias_col, qkw=None, kvkw=None):
+    """Full-size run on the GPU; the oracle is evaluated densely (fp64) on sampled query rows
+    (out, lse, dq) and sampled key columns (dk, dv; these use the GPU's lse/out for the other
+    rows, which the row samples vouch for), plus two exact invariants of softmax attention."""
+    print(f"[parity] {name}: B={B} H={H} D={D} S={S} ring={n}", flush=True)
+    gen = torch.Generator(device=device); gen.manual_seed(0)
+    mk = lambda s: (torch.randn((B, S, H, D), generator=gen, device=device) * s).to(torch.bfloat16)
+    q, k, v, do = mk(std), mk(std), mk(std), mk(1.0)
+    q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
+    out, lse = ra.ring_attention_with_lse(q, k, v, n, bias_fn=fn, bias_q_kwargs=qkw, bias_kv_kwargs=kvkw,
+                                          out_dtype=torch.float32)
+    out.backward(do.float())
+    torch.cuda.synchronize()
+    scale = 1 / math.sqrt(D)
+    # invariants (exact in real arithmetic whenever every query sees at least one key):
+    #   sum_j dv_j = sum_i do_i          (rows of P sum to one)
+    #   <q, dq> = <k, dk>                (both equal sum_ij ds_ij s_ij / scale ... per head)
+    dv_sum = v.grad.float().sum(dim=1); do_sum = do.float().sum(dim=1)
+    assert (dv_sum - do_sum).abs().max().item() <= 2e-2 * do_sum.abs().max().item() + 0.5
+    qdq = (q.detach().float() * q.grad.float()).sum(dim=(1, 3)); kdk = (k.detach().float() * k.grad.float()).sum(dim=(1, 3))
+    assert (qdq - kdk).abs().max().item() <= 2e-2 * qdq.abs().max().item() + 1.0
+    b = 0
+    heads = sorted({0, H - 1, H // 2})
+    Q, K, V, DO = (x.detach()[b].float().cpu().numpy().astype(np.float64) for x in (q, k, v, do))
+    OUT = out.detach()[b].cpu().numpy().astype(np.float64); LSE = lse[b].cpu().numpy().astype(np.float64)
+    DQ, DK, DV = (x.grad[b].float().cpu().numpy() for x in (q, k, v))
+    errs = {"out": 0.0, "lse": 0.0}
+    num = {"dq": 0.0, "dk": 0.0, "dv": 0.0}; den = {"dq": 0.0, "dk": 0.0, "dv": 0.0}
+    for h in heads:
+        for i in rows:
+            s = (K[:, h] @ Q[i, h]) * scale + bias_row(b, h, i)
+            mx = s.max(); p = np.exp(s - mx); l = p.sum()
+            o_i = (p @ V[:, h]) / l
+            errs["out"] = max(errs["out"], np.abs(OUT[i, h] - o_i).max())
+            errs["lse"] = max(errs["lse"], abs(LSE[h, i] - (mx + np.log(l))))
+            p = p / l
+            dp = V[:, h] @ DO[i, h]
+            ds = p * (dp - (p * dp).sum()) * scale
+            dq_i = ds @ K[:, h]
+            num["dq"] = max(num["dq"], np.abs(DQ[i, h] - dq_i).max()); den["dq"] = max(den["dq"], np.abs(dq_i).max())
+        delta = (OUT[:, h] * DO[:, h]).sum(axis=-1)
+        for j in cols:
+            s = (Q[:, h] @ K[j, h]) * scale + bias_col(b, h, j)
+            p = np.exp(s - LSE[h])
+            dv_j = p @ DO[:, h]
+            ds = p * (DO[:, h] @ V[j, h] - delta) * scale
+            dk_j = ds @ Q[:, h]
+            num["dv"] = max(num["dv"], np.abs(DV[j, h] - dv_j).max()); den["dv"] = max(den["dv"], np.abs(dv_j).max())
+            num["dk"] = max(num["dk"], np.abs(DK[j, h] - dk_j).max()); den["dk"] = max(den["dk"], np.abs(dk_j).max())
+    print(f"[parity] {name}: out {errs['out']:.2e} lse {errs['lse']:.2e} " +
+          " ".join(f"{kk} {num[kk] / den[kk]:.2e}" for kk in num), flush=True)
+    assert errs["out"] <= OUT_TOL and errs["lse"] <= LSE_TOL
+    for kk in num:
+        assert num[kk] / den[kk] <= GRAD_TOL, (kk, num[kk] / den[kk])
+
+
+def test_config2_full_size(device):
+    # B=2 H=16 D=128 S=8192 in 8 shards of 1024, causal with fully masked steps skipped
+    B, H, D, S, n = 2, 16, 128, 8192, 8
+    pos = np.arange(S)
+    rows = [0, 1, 1023, 1024, 4095, 4096, 5000, S - 1]
+    cols = [0, 1023, 1024, 6000, S - 1]
+    _sampled_check(device, "C2", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
+                   lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf))
+
+
+def test_config3_full_size(device):
+    # B=1 H=32 D=128 S=131072 in 8 shards of 16384, causal: the benchmark workload
+    B, H, D, S, n = 1, 32, 128, 131072, 8
+    pos = np.arange(S)
+    rows = [0, 255, 16383, 16384, 70000, S - 1]
+    cols = [0, 16383, 16384, 100000, S - 1]
+    _sampled_check(device, "C3", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
+                   lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf))
+
+
+def test_config4_full_size(device):
+    # B=1 H=16 D=128 S=32768 in 4 shards: geometric segments (mean 2048) + ALiBi 2^(-8h/H)
+    B, H, D, S, n = 1, 16, 128, 32768, 4
+    seg = R.geometric_segment_ids(0, B, S, 2048)
+    slopes = R.alibi_slopes(H)
+    pos = np.arange(S)
+    tseg = torch.from_numpy(seg).to(device)
+    rows = [0, 100, 8191, 8192, 20000, S - 1]
+    cols = [0, 8191, 8192, 30000, S - 1]
+    brow = lambda b, h, i: np.where(seg[b] == seg[b, i], 0.0, -np.inf) - slopes[h] * np.abs(i - pos)
+    _sampled_check(device, "C4", B, H, D, S, n, ra.segment_bias() + ra.alibi_bias(slopes), 1.0, rows, cols,
+                   brow, brow, {"q_segment_ids": tseg}, {"kv_segment_ids": tseg})
+
+
+def test_config5_full_size(device):
+    # B=1 H=8 D=128 S=65536 in 8 shards of 8192, causal window 4096, N(0, 0.5^2)
+    B, H, D, S, n, W = 1, 8, 128, 65536, 8, 4096
+    pos = np.arange(S)
+    rows = [0, 4095, 4096, 8191, 8192, 8193, 12287, 12288, 40000, S - 1]
+    cols = [0, 4096, 8191, 8192, 50000, S - 1]
+    _sampled_check(device, "C5", B, H, D, S, n, ra.sliding_window_bias(W), 0.5, rows, cols,
+                   lambda b, h, i: np.where((pos <= i) & (i - pos < W), 0.0, -np.inf),
+                   lambda b, h, j: np.where((pos >= j) & (pos - j < W), 0.0, -np.inf))

@@ -1,0 +1,92 @@
+"""CPU-only checks of the host-side mirror of the reference interface (no kernels run)."""
+import numpy as np
+import pytest
+import torch
+
+import ring_attention as ra
+from ring_attention import ring as rr
+from ring_attention.bias import BiasFn
+
+
+def test_public_names_match_reference_package():
+    # reference __init__.py:3 re-exports exactly these two
+    assert callable(ra.ring_attention) and callable(ra.ring_self_attention)
+
+
+def test_bias_composition_and_flags():
+    b = ra.causal_bias() + ra.segment_bias()
+    assert b.causal and b.segments and b.flags == 1 | 4
+    w = ra.sliding_window_bias(128) + ra.sliding_window_bias(64)
+    assert w.window == 64 and w.flags == 1 | 2
+    a = ra.alibi_bias([0.5, 0.25]) + ra.alibi_bias([0.5, 0.25])
+    assert torch.allclose(a.alibi_slopes, torch.tensor([1.0, 0.5]))
+    with pytest.raises(ValueError):
+        ra.causal_bias() + ra.prefix_lm_bias()  # ring.py:368-374
+    with pytest.raises(ValueError):
+        ra.sliding_window_bias(0)
+    np.testing.assert_allclose(ra.alibi_slopes(8).numpy(), [2.0 ** -(i + 1) for i in range(8)])
+
+
+def test_cpu_tensors_fail_loudly():
+    q = torch.zeros(1, 64, 1, 64)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ra.ring_attention(q, q, q, 2)
+
+
+def test_block_impl_and_bias_type_errors():
+    q = torch.zeros(1, 64, 1, 64)
+    with pytest.raises(ValueError):
+        ra.ring_attention(q, q, q, 2, block_impl="jax")  # ring.py:312 raises ValueError too
+    with pytest.raises(TypeError):
+        ra.ring_attention(q, q, q, 2, bias_fn=lambda **kw: None)
+    with pytest.raises(TypeError):
+        rr._axis_size("sp")
+    assert rr._axis_size(ra.RingAxis("sp", 8)) == 8 and rr._axis_size(("sp", 4)) == 4
+
+
+def test_ring_self_attention_argument_rules():
+    q = torch.zeros(1, 64, 1, 64)
+    pos = torch.arange(64)[None]
+    with pytest.raises(AssertionError):
+        ra.ring_self_attention(q, q, q, 2, causal=True)  # positions required (ring.py:369)
+    with pytest.raises(AssertionError):
+        ra.ring_self_attention(q, q, q, 2, causal=True, positions=pos, prefix_mask=pos)  # ring.py:370
+    with pytest.raises(AssertionError):
+        ra.ring_self_attention(q, q, q, 2, prefix_mask=pos)  # ring.py:373
+
+
+def test_ring_plan_shards_and_offsets():
+    q = torch.zeros(2, 64, 2, 64, dtype=torch.bfloat16)
+    k = torch.zeros(2, 32, 2, 64, dtype=torch.bfloat16)
+    seg_q = torch.arange(64)[None].repeat(2, 1) // 10
+    seg_k = torch.arange(32)[None].repeat(2, 1) // 10
+    plan = rr._RingPlan(q, k, 4, ra.causal_bias() + ra.segment_bias(),
+                        {"q_segment_ids": seg_q, "q_positions": torch.arange(64)[None].repeat(2, 1) + 100},
+                        {"kv_segment_ids": seg_k})
+    assert (plan.Lq, plan.Lk) == (16, 8)
+    assert plan.q_off == [100, 116, 132, 148] and plan.kv_off == [0, 8, 16, 24]
+    bb = plan.block_bias(2, 3)
+    assert bb.q_offset == 132 and bb.kv_offset == 24
+    assert torch.equal(bb.q_segment_ids, seg_q[:, 32:48].to(torch.int32))
+    assert torch.equal(bb.kv_segment_ids, seg_k[:, 24:32].to(torch.int32))
+    # shards may restart their positions, but must be consecutive inside
+    pos = torch.cat([torch.arange(16) + 7 * i for i in range(4)])[None].repeat(2, 1)
+    plan = rr._RingPlan(q, k, 4, ra.causal_bias(), {"q_positions": pos}, {})
+    assert plan.q_off == [0, 7, 14, 21]
+    with pytest.raises(NotImplementedError):
+        rr._RingPlan(q, k, 4, ra.causal_bias(), {"q_positions": pos * 2}, {})
+    with pytest.raises(ValueError):
+        rr._RingPlan(q, k, 3, None, None, None)  # 64 % 3 != 0
+    with pytest.raises(ValueError):
+        rr._RingPlan(q, k, 4, ra.segment_bias(), {"q_segment_ids": seg_q}, {})
+    with pytest.raises(ValueError):
+        rr._RingPlan(q, k, 4, ra.causal_bias(), {"bogus": seg_q}, {})
+    with pytest.raises(ValueError):
+        rr._RingPlan(q, k, 4, None, {"q_segment_ids": seg_q}, {})
+
+
+def test_shard_view_is_zero_copy():
+    x = torch.arange(2 * 8 * 3 * 4).reshape(2, 8, 3, 4)
+    s = rr._shard_bhld(x, 1, 4)
+    assert s.shape == (2, 3, 4, 4) and s.data_ptr() == x[:, 4:].data_ptr()
+    assert torch.equal(s[1, 2, 3], x[1, 7, 2])
