@@ -101,15 +101,23 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   const int* q_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.q_pre + b * bs.q_pre_sb : nullptr;
 
   f32x16 dk[NKB][DB], dv[NKB][DB];
+  {
+    // zero the accumulators THROUGH the matrix unit so that they are born in accumulation
+    // registers and stay there for the whole loop
+    bf16x8 z8;
+    f32x16 z16;
 #pragma unroll
-  for (int kb = 0; kb < NKB; ++kb)
+    for (int e = 0; e < 8; ++e) z8[e] = (bf16_t)0.f;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int r = 0; r < 16; ++r) z16[r] = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        dk[kb][db][r] = 0.f;
-        dv[kb][db][r] = 0.f;
+    for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        dk[kb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
+        dv[kb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
       }
+  }
 
   // ---- which query tiles does this workgroup visit -------------------------------------------
   const int ntiles = (a.Lq + kQTile - 1) / kQTile;
