@@ -124,8 +124,8 @@ int ra_fwd_step_check(const ra_fwd_step_params* p) {
   if ((rc = check_tensor("v", p->v))) return rc;
   if (!p->o || !p->m || !p->l) return fail(RA_ERR_NULL, "carry pointer (o, m or l) is NULL");
   if (!aligned16(p->o)) return fail(RA_ERR_ALIGN, "o is not 16-byte aligned");
-  if (!(p->sm_scale == p->sm_scale) || p->sm_scale == 0.f)
-    return fail(RA_ERR_SHAPE, "sm_scale must be a non-zero number");
+  if (!(p->sm_scale > 0.f) || p->sm_scale > 3.0e38f)
+    return fail(RA_ERR_SHAPE, "sm_scale must be a positive finite number");
   return check_bias(p->bias, p->Lq, p->Lk);
 }
 
@@ -141,8 +141,8 @@ int ra_bwd_step_check(const ra_bwd_step_params* p) {
   if (!p->dq || !p->dk || !p->dv) return fail(RA_ERR_NULL, "gradient accumulator (dq, dk or dv) is NULL");
   if (!aligned16(p->dq) || !aligned16(p->dk) || !aligned16(p->dv))
     return fail(RA_ERR_ALIGN, "gradient accumulators must be 16-byte aligned");
-  if (!(p->sm_scale == p->sm_scale) || p->sm_scale == 0.f)
-    return fail(RA_ERR_SHAPE, "sm_scale must be a non-zero number");
+  if (!(p->sm_scale > 0.f) || p->sm_scale > 3.0e38f)
+    return fail(RA_ERR_SHAPE, "sm_scale must be a positive finite number");
   return check_bias(p->bias, p->Lq, p->Lk);
 }
 

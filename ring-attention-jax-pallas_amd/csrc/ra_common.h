@@ -146,6 +146,15 @@ struct TileStage {
   }
 };
 
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l
+// (lds_base is wave-uniform and goes through M0).  Issued as inline assembly so that the
+// compiler does not guard later, unrelated LDS reads with a full vmcnt wait; completion is
+// the caller's business (s_waitcnt vmcnt(0) before the barrier that publishes the tile).
+RA_DEV void global_to_lds16(const void* gptr, const char* lds_base) {
+  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(const lds_char*)lds_base);
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
 RA_DEV bf16x8 pack8(const f32x16& p, int base) {
   bf16x8 r;
 #pragma unroll

@@ -133,7 +133,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 
   const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
   const bf16_t* vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
-  TileStage<D, kKeyTile, kFwdThreads> kst, vst;
   int seg_r = 0, pre_r = 0;
 
   auto tile_at = [&](int i, int& segbit) -> int {
@@ -145,41 +144,148 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     segbit = 0;
     return j_lo + i;
   };
-  auto issue_loads = [&](int j) {
-    kst.load(kbase, a.k.sl, j * kKeyTile, a.Lk, tid);
-    vst.load(vbase, a.v.sl, j * kKeyTile, a.Lk, tid);
+
+  // ---- global -> LDS: every wave moves 8 of a tile's 64 rows with two direct-to-LDS loads.
+  // A load instruction writes 64 lanes x 16 bytes to CONSECUTIVE LDS addresses, i.e. lane l
+  // fills physical chunk l%CPR of row l/CPR; the XOR layout is obtained by letting that lane
+  // fetch logical chunk (l%CPR) ^ f(row) from global memory instead.
+  constexpr int CPR = D / 8;            // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;         // rows per load instruction
+  constexpr int NLD = 8 / RPI;          // load instructions per wave per tile
+  int ld_row[NLD];
+  long long ld_koff[NLD], ld_voff[NLD];
+#pragma unroll
+  for (int t = 0; t < NLD; ++t) {
+    const int rrow = 8 * wave + RPI * t + lane / CPR;
+    const int pc = lane % CPR;
+    const int lc = (tile_off<D>(rrow, pc) - rrow * (D * 2)) >> 4;  // logical chunk stored at pc
+    ld_row[t] = rrow;
+    ld_koff[t] = lc * 8;
+    ld_voff[t] = lc * 8;
+  }
+  auto issue_k = [&](int j, int buf) {
+    const int k0 = j * kKeyTile;
+#pragma unroll
+    for (int t = 0; t < NLD; ++t) {
+      const int gr = min(k0 + ld_row[t], a.Lk - 1);
+      const bf16_t* src = kbase + (long long)gr * a.k.sl + ld_koff[t];
+      global_to_lds16(src, s_k[buf] + (8 * wave + RPI * t) * (D * 2));
+    }
     if (GENERAL && tid < kKeyTile) {
-      int kk = min(j * kKeyTile + tid, a.Lk - 1);
+      int kk = min(k0 + tid, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
     }
   };
-
-  int segbit = 0;
-  if (n_act > 0) issue_loads(tile_at(0, segbit));
-
-  for (int i = 0; i < n_act; ++i) {
-    const int buf = i & 1;
-    kst.store(s_k[buf], tid);
-    vst.store(s_v[buf], tid);
+  auto issue_v = [&](int j, int buf) {
+    const int k0 = j * kKeyTile;
+#pragma unroll
+    for (int t = 0; t < NLD; ++t) {
+      const int gr = min(k0 + ld_row[t], a.Lk - 1);
+      const bf16_t* src = vbase + (long long)gr * a.v.sl + ld_voff[t];
+      global_to_lds16(src, s_v[buf] + (8 * wave + RPI * t) * (D * 2));
+    }
+  };
+  // pair p = (K tile p, V tile p-1) -> LDS buffer p & 1
+  const int n = n_act;
+  int sb_unused;
+  auto issue_pair = [&](int pidx) {
+    if (pidx < n) issue_k(tile_at(pidx, sb_unused), pidx & 1);
+    if (pidx >= 1 && pidx - 1 < n) issue_v(tile_at(pidx - 1, sb_unused), pidx & 1);
+  };
+  auto store_ids = [&](int buf) {
     if (GENERAL && tid < kKeyTile) {
       s_seg[buf][tid] = seg_r;
       s_pre[buf][tid] = pre_r;
     }
-    __syncthreads();
-    int cur_segbit;
-    const int j = tile_at(i, cur_segbit);
-    if (i + 1 < n_act) {
-      int nb;
-      issue_loads(tile_at(i + 1, nb));
-    }
+  };
 
-    // ---- classify this wave's 32 x 64 rectangle ------------------------------------------
-    const int kt0 = j * kKeyTile;
+  // ---- main loop: two wave groups in opposite phases -------------------------------------------
+  // Waves 0-3 (group 0) and 4-7 (group 1) share the four SIMDs pairwise.  Time is cut into
+  // slots separated by workgroup barriers.  In every slot one group runs a MATRIX phase (PV of
+  // the previous tile, then S of the next one: 32 MFMAs fed by software-pipelined LDS reads)
+  // while the other runs the VECTOR phase of the tile in between (bias, row statistics, exp2,
+  // bf16 packing), so the matrix unit and the vector ALU of a SIMD work at the same time.
+  // Group 0 runs matrix phase i in slot 2i and vector phase i in slot 2i+1; group 1 is one slot
+  // behind.  Pair p is fetched during slots 2p-2 and 2p-1 and consumed in slots 2p and 2p+1.
+  const int grp = wave >> 2;
+  issue_pair(0);
+  store_ids(0);
+  __builtin_amdgcn_s_waitcnt(0);  // also: carry and Q operand loads have landed
+  __syncthreads();
+
+  f32x16 sacc[2];
+  bf16x8 pfrag[4];
+  bool s_valid = false, p_valid = false;
+  float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
+  const bool wave_on = qw < a.Lq;
+
+  constexpr int PF = 6;  // LDS operand fetches kept in flight ahead of the MFMA that uses them
+  auto matrix_phase = [&](int i, int buf) {
+    __builtin_amdgcn_s_setprio(2);
+    const char* vt = s_v[buf];
+    const char* kt = s_k[buf];
+    if (p_valid) {
+      // O^T += V^T P^T : op = (kb, ks, db)
+      bf16x8 fr[16];
+#pragma unroll
+      for (int op = 0; op < PF; ++op)
+        fr[op] = frag_tr<D>(vt, 32 * (op / (2 * DB)) + 16 * ((op / DB) & 1), 32 * (op % DB), lane);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int op = 0; op < 4 * DB; ++op) {
+        if (op + PF < 4 * DB) {
+          const int o2 = op + PF;
+          fr[o2] = frag_tr<D>(vt, 32 * (o2 / (2 * DB)) + 16 * ((o2 / DB) & 1), 32 * (o2 % DB), lane);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      p_valid = false;
+    }
+    s_valid = false;
+    if (i < n && wave_on) {
+      int segbit_i;
+      const int kt0 = tile_at(i, segbit_i) * kKeyTile;
+      const int cls = (flags & RA_BIAS_PREFIX)
+                          ? 2
+                          : classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31,
+                                         bs.kv_off + kt0, bs.kv_off + kt0 + kKeyTile - 1);
+      if (!(cls & 1)) {
+        s_valid = true;
+        // S^T = K Q^T : op = (ks, kb)
+        bf16x8 fr[2 * KS];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          sacc[0][r] = 0.f;
+          sacc[1][r] = 0.f;
+        }
+#pragma unroll
+        for (int op = 0; op < PF; ++op) fr[op] = frag_nat<D>(kt, 32 * (op & 1) + l32, op >> 1, g);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int op = 0; op < 2 * KS; ++op) {
+          if (op + PF < 2 * KS) {
+            const int o2 = op + PF;
+            fr[o2] = frag_nat<D>(kt, 32 * (o2 & 1) + l32, o2 >> 1, g);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          sacc[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], sacc[op & 1], 0, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    __builtin_amdgcn_s_setprio(0);
+  };
+
+  auto vector_phase = [&](int i, int buf) {
+    if (!s_valid) return;
+    int cur_segbit;
+    const int kt0 = tile_at(i, cur_segbit) * kKeyTile;
     const int qlo = bs.q_off + qw, qhi = qlo + 31;
     const int klo = bs.kv_off + kt0, khi = klo + kKeyTile - 1;
     const int cls = (flags & RA_BIAS_PREFIX) ? 2 : classify_pos(flags, bs.window, qlo, qhi, klo, khi);
-    if ((cls & 1) || qw >= a.Lq) continue;
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
@@ -188,68 +294,107 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
-    const bool ragged = kt0 + kKeyTile > a.Lk;
-    const bool need_bias = tb.flags != 0 || ragged;
-
-    // ---- S^T = K Q^T ---------------------------------------------------------------------
-    f32x16 sacc[2];
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        bf16x8 kf = frag_nat<D>(s_k[buf], 32 * kb + l32, s, g);
-        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[s], sacc[kb], 0, 0, 0);
-      }
-    }
-    // ---- scale, bias, row statistics -------------------------------------------------------
+    const bool need_bias = tb.flags != 0 || (kt0 + kKeyTile > a.Lk);
     float mx = RA_NEG_INF;
+    if (need_bias) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+      for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[kb][r] *= a.scale2;
-      if (need_bias) {
+        for (int r = 0; r < 16; ++r) sacc[kb][r] *= a.scale2;
         const int var0 = kt0 + 32 * kb + 4 * g;
         tb.var_limit = a.Lk - var0;
         const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
         apply_bias<true>(sacc[kb], tb, rel0, q_seg, q_pre, &s_seg[buf][32 * kb + 4 * g],
                          &s_pre[buf][32 * kb + 4 * g]);
-      }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
+      }
+      mx = half_max(mx);
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
+      mx = half_max(mx) * a.scale2;  // scale2 > 0: the maximum commutes with the scaling
     }
-    mx = half_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = (m_new == RA_NEG_INF) ? 0.f : m_new;
-    const float corr = fast_exp2(m_run - m_safe);
-    m_run = m_new;
+    m_true = fmaxf(m_true, mx);
+    // The exponent reference only moves when some row's maximum grew by more than 2^8; until
+    // then probabilities are taken relative to the old reference (they stay below 256,
+    // harmless in fp32 / bf16) and the 64-register rescale of O is skipped.
+    if (__any(mx > m_run + 8.0f)) {
+      const float m_new = fmaxf(m_run, mx);
+      const float m_safe_new = (m_new == RA_NEG_INF) ? 0.f : m_new;
+      const float corr = fast_exp2(m_run - m_safe_new);
+      m_run = m_new;
+      l_run *= corr;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= corr;
+    }
+    const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
     float rs = 0.f;
+    if (need_bias) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float p = fast_exp2(sacc[kb][r] - m_safe);
-        sacc[kb][r] = p;
-        rs += p;
-      }
-    l_run = l_run * corr + rs;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[db][r] *= corr;
-    // ---- O^T += V^T P^T -----------------------------------------------------------------
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const bf16x8 pf = pack8(sacc[kb], 8 * ks);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          bf16x8 vf = frag_tr<D>(s_v[buf], 32 * kb + 16 * ks, 32 * db, lane);
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf, oacc[db], 0, 0, 0);
+        for (int r = 0; r < 16; ++r) {
+          float p = fast_exp2(sacc[kb][r] + neg_m);
+          sacc[kb][r] = p;
+          rs += p;
         }
-      }
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float p = fast_exp2(fmaf(sacc[kb][r], a.scale2, neg_m));
+          sacc[kb][r] = p;
+          rs += p;
+        }
+    }
+    l_run += rs;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) pfrag[2 * kb + ks] = pack8(sacc[kb], 8 * ks);
+    p_valid = true;
+    s_valid = false;
+  };
+
+  if (grp == 1) {  // slot 0 of group 1: nothing to compute yet, but its share of pair 1 is due
+    issue_pair(1);
+    __syncthreads();
+  }
+  for (int i = 0; i <= n; ++i) {
+    const int buf = i & 1;
+    // matrix phase i  (group 0: slot 2i, group 1: slot 2i+1)
+    if (grp == 0) issue_pair(i + 1);
+    matrix_phase(i, buf);
+    if (grp == 1) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): pair i+1 complete
+    __syncthreads();
+    // vector phase i  (group 0: slot 2i+1, group 1: slot 2i+2)
+    if (grp == 1) issue_pair(i + 2);
+    vector_phase(i, buf);
+    if (grp == 0) {
+      store_ids((i + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): pair i+1 complete
+    }
+    if (i < n || grp == 0) __syncthreads();
+  }
+
+  // bring the carry back to the exact maximum
+  {
+    const float m_safe = (m_true == RA_NEG_INF) ? 0.f : m_true;
+    const float f = fast_exp2(m_run - m_safe);  // 1 where the reference is exact, 0 for empty rows
+    if (__any(m_run != m_true)) {
+      l_run *= f;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[db][r] *= f;
+    }
+    m_run = m_true;
   }
 
   // ---- write the carry back ------------------------------------------------------------------
