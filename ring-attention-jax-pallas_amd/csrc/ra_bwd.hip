@@ -14,7 +14,7 @@
 
 namespace ra {
 
-constexpr int kMaxListTiles = 2048;
+constexpr int kBwdMaxListTiles = 2048;
 
 // ------------------------------------------------------------------------------------------------
 // delta
@@ -63,8 +63,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   __shared__ __attribute__((aligned(16))) float s_delta[2][kQTile];
   __shared__ __attribute__((aligned(16))) int s_seg[2][kQTile];
   __shared__ __attribute__((aligned(16))) int s_pre[2][kQTile];
-  __shared__ unsigned short s_list[GENERAL ? kMaxListTiles : 1];
-  __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
+  __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
+  __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[12];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -324,20 +324,20 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 // ------------------------------------------------------------------------------------------------
 constexpr int kDqThreads = 512;
 constexpr int kDqRows = 256;
-constexpr int kKeyTile = 64;
+constexpr int kDqKeyTile = 64;
 
 template <int D, bool GENERAL>
 __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
-  constexpr int TILE_BYTES = kKeyTile * D * 2;
+  constexpr int TILE_BYTES = kDqKeyTile * D * 2;
 
   __shared__ __attribute__((aligned(16))) char s_k[2][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char s_v[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) int s_seg[2][kKeyTile];
-  __shared__ __attribute__((aligned(16))) int s_pre[2][kKeyTile];
-  __shared__ unsigned short s_list[GENERAL ? kMaxListTiles : 1];
-  __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
+  __shared__ __attribute__((aligned(16))) int s_seg[2][kDqKeyTile];
+  __shared__ __attribute__((aligned(16))) int s_pre[2][kDqKeyTile];
+  __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
+  __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[20];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -384,10 +384,10 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.kv_seg + b * bs.kv_seg_sb : nullptr;
   const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.kv_pre + b * bs.kv_pre_sb : nullptr;
 
-  const int ntiles = (a.Lk + kKeyTile - 1) / kKeyTile;
+  const int ntiles = (a.Lk + kDqKeyTile - 1) / kDqKeyTile;
   const int q_rows_hi = min(q0 + kDqRows, a.Lq) - 1;
   int j_lo, j_hi;
-  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, bs.kv_off, ntiles, kKeyTile,
+  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, bs.kv_off, ntiles, kDqKeyTile,
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
@@ -409,8 +409,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     }
     for (int j = j_lo + tid; j < j_hi; j += kDqThreads) {
       int kmin = 0x7fffffff, kmax = (int)0x80000000;
-      const int kend = min((j + 1) * kKeyTile, a.Lk);
-      for (int kk = j * kKeyTile; kk < kend; ++kk) {
+      const int kend = min((j + 1) * kDqKeyTile, a.Lk);
+      for (int kk = j * kDqKeyTile; kk < kend; ++kk) {
         int sid = kv_seg[kk];
         kmin = min(kmin, sid);
         kmax = max(kmax, sid);
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
 
   const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
   const bf16_t* vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
-  TileStage<D, kKeyTile, kDqThreads> kst, vst;
+  TileStage<D, kDqKeyTile, kDqThreads> kst, vst;
   int seg_r = 0, pre_r = 0;
 
   auto tile_at = [&](int i, int& segbit) -> int {
@@ -450,10 +450,10 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     return j_lo + i;
   };
   auto issue_loads = [&](int j) {
-    kst.load(kbase, a.k.sl, j * kKeyTile, a.Lk, tid);
-    vst.load(vbase, a.v.sl, j * kKeyTile, a.Lk, tid);
-    if (GENERAL && tid < kKeyTile) {
-      int kk = min(j * kKeyTile + tid, a.Lk - 1);
+    kst.load(kbase, a.k.sl, j * kDqKeyTile, a.Lk, tid);
+    vst.load(vbase, a.v.sl, j * kDqKeyTile, a.Lk, tid);
+    if (GENERAL && tid < kDqKeyTile) {
+      int kk = min(j * kDqKeyTile + tid, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
     }
@@ -466,7 +466,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     const int buf = i & 1;
     kst.store(s_k[buf], tid);
     vst.store(s_v[buf], tid);
-    if (GENERAL && tid < kKeyTile) {
+    if (GENERAL && tid < kDqKeyTile) {
       s_seg[buf][tid] = seg_r;
       s_pre[buf][tid] = pre_r;
     }
@@ -478,7 +478,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       issue_loads(tile_at(i + 1, nb));
     }
     if (qw >= a.Lq) continue;
-    const int kt0 = j * kKeyTile;
+    const int kt0 = j * kDqKeyTile;
     const int qlo = bs.q_off + qw, qhi = qlo + 31;
 
 #pragma unroll

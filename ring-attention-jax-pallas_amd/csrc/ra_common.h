@@ -19,6 +19,29 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 #define RA_DEV __device__ __forceinline__
 
+// Optional in-kernel phase timing (build with -DRA_PROFILE): every wave accumulates, in scalar
+// registers, the cycles spent between consecutive marks; waves 0 and 4 of workgroup 0 write
+// the sums to g_prof[wave/4][segment] when the kernel ends.  Compiles to nothing otherwise.
+#ifdef RA_PROFILE
+__device__ unsigned int g_prof[2][16];
+#define RA_PROF_DECL unsigned int prof_seg[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long prof_t = __builtin_readcyclecounter();
+#define RA_PROF_MARK(iter, id)                                         \
+  do {                                                                 \
+    unsigned long long t_ = __builtin_readcyclecounter();              \
+    prof_seg[id] += (unsigned int)(t_ - prof_t);                       \
+    prof_t = t_;                                                       \
+  } while (0)
+#define RA_PROF_DUMP                                                   \
+  do {                                                                 \
+    if (blockIdx.x == 0 && (threadIdx.x & 255) == 0)                   \
+      for (int i_ = 0; i_ < 8; ++i_) g_prof[threadIdx.x >> 8][i_] = prof_seg[i_]; \
+  } while (0)
+#else
+#define RA_PROF_DECL
+#define RA_PROF_MARK(iter, id) do { } while (0)
+#define RA_PROF_DUMP do { } while (0)
+#endif
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 #define RA_NEG_INF (-__builtin_inff())

@@ -7,7 +7,13 @@
 // exchange with lane^32, the rescale of the running output is a per-lane scalar, and the
 // bf16 probabilities are already laid out as the B operand of O^T = V^T P^T, whose A
 // operand comes from the V tile through the transposing LDS read.
+#include <type_traits>
+
 #include "ra_launch.h"
+
+#ifndef RA_ABLATE
+#define RA_ABLATE 0  // timing experiments only: bit mask of loop parts to leave out
+#endif
 
 namespace ra {
 
@@ -152,8 +158,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   constexpr int CPR = D / 8;            // 16-byte chunks per row
   constexpr int RPI = 64 / CPR;         // rows per load instruction
   constexpr int NLD = 8 / RPI;          // load instructions per wave per tile
-  int ld_row[NLD];
-  long long ld_koff[NLD], ld_voff[NLD];
+  int ld_row[NLD], ld_koff[NLD];
 #pragma unroll
   for (int t = 0; t < NLD; ++t) {
     const int rrow = 8 * wave + RPI * t + lane / CPR;
@@ -161,7 +166,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     const int lc = (tile_off<D>(rrow, pc) - rrow * (D * 2)) >> 4;  // logical chunk stored at pc
     ld_row[t] = rrow;
     ld_koff[t] = lc * 8;
-    ld_voff[t] = lc * 8;
   }
   auto issue_k = [&](int j, int buf) {
     const int k0 = j * kKeyTile;
@@ -182,17 +186,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 #pragma unroll
     for (int t = 0; t < NLD; ++t) {
       const int gr = min(k0 + ld_row[t], a.Lk - 1);
-      const bf16_t* src = vbase + (long long)gr * a.v.sl + ld_voff[t];
+      const bf16_t* src = vbase + (long long)gr * a.v.sl + ld_koff[t];
       global_to_lds16(src, s_v[buf] + (8 * wave + RPI * t) * (D * 2));
     }
   };
-  // pair p = (K tile p, V tile p-1) -> LDS buffer p & 1
   const int n = n_act;
   int sb_unused;
-  auto issue_pair = [&](int pidx) {
-    if (pidx < n) issue_k(tile_at(pidx, sb_unused), pidx & 1);
-    if (pidx >= 1 && pidx - 1 < n) issue_v(tile_at(pidx - 1, sb_unused), pidx & 1);
-  };
   auto store_ids = [&](int buf) {
     if (GENERAL && tid < kKeyTile) {
       s_seg[buf][tid] = seg_r;
@@ -200,127 +199,142 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     }
   };
 
-  // ---- main loop: two wave groups in opposite phases -------------------------------------------
-  // Waves 0-3 (group 0) and 4-7 (group 1) share the four SIMDs pairwise.  Time is cut into
-  // slots separated by workgroup barriers.  In every slot one group runs a MATRIX phase (PV of
-  // the previous tile, then S of the next one: 32 MFMAs fed by software-pipelined LDS reads)
-  // while the other runs the VECTOR phase of the tile in between (bias, row statistics, exp2,
-  // bf16 packing), so the matrix unit and the vector ALU of a SIMD work at the same time.
-  // Group 0 runs matrix phase i in slot 2i and vector phase i in slot 2i+1; group 1 is one slot
-  // behind.  Pair p is fetched during slots 2p-2 and 2p-1 and consumed in slots 2p and 2p+1.
-  const int grp = wave >> 2;
-  issue_pair(0);
-  store_ids(0);
-  __builtin_amdgcn_s_waitcnt(0);  // also: carry and Q operand loads have landed
+  // ---- main loop ----------------------------------------------------------------------------------
+  // The matrix unit runs ahead of the vector ALU inside every wave: while the 16 MFMAs of
+  // S(i+1) = K_{i+1} Q^T are in flight, the same wave turns S(i) into probabilities (exp2, row
+  // sum, bf16 packing), and while the 16 MFMAs of O += P(i) V_i run it takes the row maximum of
+  // S(i+1).  Vector instructions issued by the wave that owns the MFMA in flight slip into its
+  // shadow; the second wave of the SIMD covers LDS and barrier latency.
+  // LDS: K tile j lives in s_k[j & 1], V tile j in s_v[j & 1].  Iteration i reads K_{i+1} and V_i
+  // and, right after the barrier that ends iteration i-1, refills the two buffers nobody reads
+  // any more with K_{i+2} and V_{i+1}.
+  const bool wave_on = qw < a.Lq;
+  if (n > 0) {
+    issue_k(tile_at(0, sb_unused), 0);
+    store_ids(0);
+    issue_v(tile_at(0, sb_unused), 0);
+  }
+  if (n > 1) {
+    issue_k(tile_at(1, sb_unused), 1);
+    store_ids(1);
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // tiles, carry and Q operands have landed
   __syncthreads();
 
-  f32x16 sacc[2];
-  bf16x8 pfrag[4];
-  bool s_valid = false, p_valid = false;
   float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
-  const bool wave_on = qw < a.Lq;
+  RA_PROF_DECL
+  constexpr int PF = 3;  // LDS operand fetches kept in flight ahead of the MFMA that uses them
 
-  constexpr int PF = 6;  // LDS operand fetches kept in flight ahead of the MFMA that uses them
-  auto matrix_phase = [&](int i, int buf) {
-    __builtin_amdgcn_s_setprio(2);
-    const char* vt = s_v[buf];
-    const char* kt = s_k[buf];
-    if (p_valid) {
-      // O^T += V^T P^T : op = (kb, ks, db)
-      bf16x8 fr[16];
-#pragma unroll
-      for (int op = 0; op < PF; ++op)
-        fr[op] = frag_tr<D>(vt, 32 * (op / (2 * DB)) + 16 * ((op / DB) & 1), 32 * (op % DB), lane);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int op = 0; op < 4 * DB; ++op) {
-        if (op + PF < 4 * DB) {
-          const int o2 = op + PF;
-          fr[o2] = frag_tr<D>(vt, 32 * (o2 / (2 * DB)) + 16 * ((o2 / DB) & 1), 32 * (o2 % DB), lane);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      p_valid = false;
-    }
-    s_valid = false;
-    if (i < n && wave_on) {
-      int segbit_i;
-      const int kt0 = tile_at(i, segbit_i) * kKeyTile;
-      const int cls = (flags & RA_BIAS_PREFIX)
-                          ? 2
-                          : classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31,
-                                         bs.kv_off + kt0, bs.kv_off + kt0 + kKeyTile - 1);
-      if (!(cls & 1)) {
-        s_valid = true;
-        // S^T = K Q^T : op = (ks, kb)
-        bf16x8 fr[2 * KS];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          sacc[0][r] = 0.f;
-          sacc[1][r] = 0.f;
-        }
-#pragma unroll
-        for (int op = 0; op < PF; ++op) fr[op] = frag_nat<D>(kt, 32 * (op & 1) + l32, op >> 1, g);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int op = 0; op < 2 * KS; ++op) {
-          if (op + PF < 2 * KS) {
-            const int o2 = op + PF;
-            fr[o2] = frag_nat<D>(kt, 32 * (o2 & 1) + l32, o2 >> 1, g);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-          sacc[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], sacc[op & 1], 0, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-    }
-    __builtin_amdgcn_s_setprio(0);
+  // positional class of this wave's 32 x 64 rectangle of tile index i
+  auto tile_class = [&](int i, int& kt0, int& segbit) -> int {
+    kt0 = tile_at(i, segbit) * kKeyTile;
+    if (flags & RA_BIAS_PREFIX) return 2;
+    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off + kt0,
+                        bs.kv_off + kt0 + kKeyTile - 1);
   };
-
-  auto vector_phase = [&](int i, int buf) {
-    if (!s_valid) return;
-    int cur_segbit;
-    const int kt0 = tile_at(i, cur_segbit) * kKeyTile;
-    const int qlo = bs.q_off + qw, qhi = qlo + 31;
-    const int klo = bs.kv_off + kt0, khi = klo + kKeyTile - 1;
-    const int cls = (flags & RA_BIAS_PREFIX) ? 2 : classify_pos(flags, bs.window, qlo, qhi, klo, khi);
+  // Per-lane LDS byte offsets of the operand fetches.  Everything that changes from one MFMA
+  // to the next (tile buffer, 32-key block, 16-key step) is a multiple of 16 rows, which the
+  // XOR layout leaves alone, so it folds into the instruction's immediate offset field.
+  int koff[KS];
+#pragma unroll
+  for (int ss = 0; ss < KS; ++ss) koff[ss] = tile_off<D>(l32, 2 * ss + g);
+  int voff[DB][2];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int hh2 = 0; hh2 < 2; ++hh2) {
+      const int j = lane & 15;
+      const int vrow = 4 * g + (j >> 2) + 8 * hh2;
+      const int vcol = 32 * db + 16 * ((lane >> 4) & 1) + 4 * (j & 3);
+      voff[db][hh2] = tile_off<D>(vrow, vcol >> 3) + ((vcol & 4) << 1);
+    }
+  constexpr int ROWB = D * 2;
+  auto s_op_frag = [&](const char* kt, int op) {
+    if (RA_ABLATE & 32) return qf[op >> 1];
+    return *(const bf16x8*)(kt + (32 * (op & 1)) * ROWB + koff[op >> 1]);
+  };
+  auto pv_op_frag = [&](const char* vt, int op) {
+    if (RA_ABLATE & 64) return qf[op % KS];
+    const int cofs = (32 * (op / (2 * DB)) + 16 * ((op / DB) & 1)) * ROWB;
+    const lds_char* p0 = (const lds_char*)(vt + cofs + voff[op % DB][0]);
+    const lds_char* p1 = (const lds_char*)(vt + cofs + voff[op % DB][1]);
+    bf16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p0);
+    bf16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p1);
+    return __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  // S = K Q^T for one tile, nothing interleaved
+  auto compute_s = [&](f32x16 (&S)[2], const char* kt) {
+    bf16x8 fr[2 * KS];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      S[0][r] = 0.f;
+      S[1][r] = 0.f;
+    }
+#pragma unroll
+    for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 2 * KS; ++op) {
+      if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
+      S[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], S[op & 1], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto compute_pv = [&](const bf16x8 (&pf)[4], const char* vt) {
+    bf16x8 fr[4 * DB];
+#pragma unroll
+    for (int op = 0; op < PF; ++op) fr[op] = pv_op_frag(vt, op);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 4 * DB; ++op) {
+      if (op + PF < 4 * DB) fr[op + PF] = pv_op_frag(vt, op + PF);
+      oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pf[op / DB], oacc[op % DB], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto raw_rowmax = [&](const f32x16 (&S)[2]) -> float {
+    float mx = RA_NEG_INF;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
+    return half_max(mx) * a.scale2;  // scale2 > 0: the maximum commutes with the scaling
+  };
+  auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
+    bool nb = (cls & 2) || (kt0 + kKeyTile > a.Lk);
+    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
+    return nb;
+  };
+  // scale + bias with the id arrays of LDS slot `ids_buf`; returns the row maximum
+  auto prepare = [&](f32x16 (&S)[2], int kt0, int segbit, int cls, int ids_buf) -> float {
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
       tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
-      if (cur_segbit) tb.flags |= RA_BIAS_SEGMENT;
+      if (segbit) tb.flags |= RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
-    const bool need_bias = tb.flags != 0 || (kt0 + kKeyTile > a.Lk);
     float mx = RA_NEG_INF;
-    if (need_bias) {
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
+    for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[kb][r] *= a.scale2;
-        const int var0 = kt0 + 32 * kb + 4 * g;
-        tb.var_limit = a.Lk - var0;
-        const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
-        apply_bias<true>(sacc[kb], tb, rel0, q_seg, q_pre, &s_seg[buf][32 * kb + 4 * g],
-                         &s_pre[buf][32 * kb + 4 * g]);
+      for (int r = 0; r < 16; ++r) S[kb][r] *= a.scale2;
+      const int var0 = kt0 + 32 * kb + 4 * g;
+      tb.var_limit = a.Lk - var0;
+      const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
+      apply_bias<true>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
+                       &s_pre[ids_buf][32 * kb + 4 * g]);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
-      }
-      mx = half_max(mx);
-    } else {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kb][r]);
-      mx = half_max(mx) * a.scale2;  // scale2 > 0: the maximum commutes with the scaling
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
     }
+    return half_max(mx);
+  };
+  // move the exponent reference if some row's maximum outgrew it by more than 2^8; until then
+  // probabilities are taken relative to the old reference (they stay below 256, harmless in
+  // fp32 / bf16) and the 64-register rescale of O is skipped
+  auto update_reference = [&](float mx) {
     m_true = fmaxf(m_true, mx);
-    // The exponent reference only moves when some row's maximum grew by more than 2^8; until
-    // then probabilities are taken relative to the old reference (they stay below 256,
-    // harmless in fp32 / bf16) and the 64-register rescale of O is skipped.
     if (__any(mx > m_run + 8.0f)) {
       const float m_new = fmaxf(m_run, mx);
       const float m_safe_new = (m_new == RA_NEG_INF) ? 0.f : m_new;
@@ -332,57 +346,144 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] *= corr;
     }
-    const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
-    float rs = 0.f;
-    if (need_bias) {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float p = fast_exp2(sacc[kb][r] + neg_m);
-          sacc[kb][r] = p;
-          rs += p;
-        }
-    } else {
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          float p = fast_exp2(fmaf(sacc[kb][r], a.scale2, neg_m));
-          sacc[kb][r] = p;
-          rs += p;
-        }
-    }
-    l_run += rs;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) pfrag[2 * kb + ks] = pack8(sacc[kb], 8 * ks);
-    p_valid = true;
-    s_valid = false;
   };
 
-  if (grp == 1) {  // slot 0 of group 1: nothing to compute yet, but its share of pair 1 is due
-    issue_pair(1);
-    __syncthreads();
-  }
-  for (int i = 0; i <= n; ++i) {
-    const int buf = i & 1;
-    // matrix phase i  (group 0: slot 2i, group 1: slot 2i+1)
-    if (grp == 0) issue_pair(i + 1);
-    matrix_phase(i, buf);
-    if (grp == 1) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): pair i+1 complete
-    __syncthreads();
-    // vector phase i  (group 0: slot 2i+1, group 1: slot 2i+2)
-    if (grp == 1) issue_pair(i + 2);
-    vector_phase(i, buf);
-    if (grp == 0) {
-      store_ids((i + 1) & 1);
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): pair i+1 complete
+  // per-tile state handed from one iteration to the next
+  f32x16 sa[2], sb[2];
+  bool cur_valid = false, cur_scaled = false;
+  float cur_mx = RA_NEG_INF;
+  if (n > 0 && wave_on) {
+    int kt0, segbit;
+    const int cls = tile_class(0, kt0, segbit);
+    if (!(cls & 1)) {
+      cur_valid = true;
+      compute_s(sa, s_k[0]);
+      cur_scaled = needs_bias(kt0, segbit, cls);
+      cur_mx = cur_scaled ? prepare(sa, kt0, segbit, cls, 0) : raw_rowmax(sa);
     }
-    if (i < n || grp == 0) __syncthreads();
   }
 
+  // one iteration; SC holds S(i) on entry, SN receives S(i+1)
+  auto iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
+    constexpr int PAR = decltype(parity)::value;  // i & 1, known at compile time
+    RA_PROF_MARK(i, 1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of K_{i+1}, V_i is in LDS
+    if (!(RA_ABLATE & 8)) __syncthreads();
+    RA_PROF_MARK(i, 2);
+    if (!(RA_ABLATE & 1)) {
+      if (i + 2 < n) issue_k(tile_at(i + 2, sb_unused), PAR);
+      if (i + 1 < n) issue_v(tile_at(i + 1, sb_unused), PAR ^ 1);
+    }
+    const char* kt = s_k[PAR ^ 1];
+    const char* vt = s_v[PAR];
+    int nkt0 = 0, nsegbit = 0, ncls = 1;
+    bool nxt_valid = false;
+    if (i + 1 < n && wave_on) {
+      ncls = tile_class(i + 1, nkt0, nsegbit);
+      nxt_valid = !(ncls & 1);
+    }
+    const bool nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
+    float nxt_mx = RA_NEG_INF;
+    bf16x8 pfrag[4];
+    if (cur_valid) update_reference(cur_mx);
+    const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
+
+    RA_PROF_MARK(i, 3);
+    if (cur_valid && nxt_valid && !cur_scaled) {
+      // ---- fused path: S(i+1) MFMAs with the exp2 / sum / pack of tile i in their shadow -------
+      float rs0 = 0.f, rs1 = 0.f;
+      {
+        bf16x8 fr[2 * KS];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          SN[0][r] = 0.f;
+          SN[1][r] = 0.f;
+        }
+#pragma unroll
+        for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
+        __builtin_amdgcn_sched_barrier(0);
+        constexpr int EPO = 32 / (2 * KS);  // score elements converted per MFMA
+#pragma unroll
+        for (int op = 0; op < 2 * KS; ++op) {
+          if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
+          if (!(RA_ABLATE & 16)) SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
+          else SN[op & 1][op >> 1] += (float)fr[op][0];
+#pragma unroll
+          for (int e = 0; e < ((RA_ABLATE & 2) ? 0 : EPO); e += 2) {
+            const int el = op * EPO + e;  // 0..31 over (kb, r)
+            const int kb = el >> 4, r = el & 15;
+            const float p0 = fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
+            const float p1 = fast_exp2(fmaf(SC[kb][r + 1], a.scale2, neg_m));
+            rs0 += p0;
+            rs1 += p1;
+            pfrag[2 * kb + (r >> 3)][r & 7] = (bf16_t)p0;
+            pfrag[2 * kb + (r >> 3)][(r & 7) + 1] = (bf16_t)p1;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      l_run += rs0 + rs1;
+      RA_PROF_MARK(i, 4);
+      // ---- O += P(i) V_i with the row maximum of S(i+1) in the shadow ---------------------------
+      {
+        bf16x8 fr[4 * DB];
+        float mx0 = RA_NEG_INF, mx1 = RA_NEG_INF;
+#pragma unroll
+        for (int op = 0; op < PF; ++op) fr[op] = pv_op_frag(vt, op);
+        __builtin_amdgcn_sched_barrier(0);
+        constexpr int EPO = 32 / (4 * DB);
+#pragma unroll
+        for (int op = 0; op < 4 * DB; ++op) {
+          if (op + PF < 4 * DB) fr[op + PF] = pv_op_frag(vt, op + PF);
+          if (!(RA_ABLATE & 4)) oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
+          else oacc[op % DB][op / DB] += (float)fr[op][0] * (float)pfrag[op / DB][0];
+#pragma unroll
+          for (int e = 0; e < EPO; e += 2) {
+            const int el = op * EPO + e;
+            mx0 = fmaxf(mx0, SN[el >> 4][el & 15]);
+            mx1 = fmaxf(mx1, SN[el >> 4][(el & 15) + 1]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        nxt_mx = half_max(fmaxf(mx0, mx1)) * a.scale2;
+      }
+      RA_PROF_MARK(i, 5);
+    } else {
+      // ---- generic path (first / last / masked / biased tiles): same work, not interleaved -----
+      if (nxt_valid) compute_s(SN, kt);
+      if (cur_valid) {
+        float rs = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float p = cur_scaled ? fast_exp2(SC[kb][r] + neg_m) : fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
+            SC[kb][r] = p;
+            rs += p;
+          }
+        l_run += rs;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int ks = 0; ks < 2; ++ks) pfrag[2 * kb + ks] = pack8(SC[kb], 8 * ks);
+        compute_pv(pfrag, vt);
+      }
+      if (nxt_valid && !nxt_scaled) nxt_mx = raw_rowmax(SN);
+    }
+    RA_PROF_MARK(i, 6);
+    if (nxt_scaled) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, PAR ^ 1);
+    if (i + 2 < n) store_ids(PAR);
+    cur_valid = nxt_valid;
+    cur_scaled = nxt_scaled;
+    cur_mx = nxt_mx;
+  };
+
+  for (int i = 0; i < n; i += 2) {
+    iteration(std::integral_constant<int, 0>{}, i, sa, sb);
+    if (i + 1 < n) iteration(std::integral_constant<int, 1>{}, i + 1, sb, sa);
+  }
+
+  RA_PROF_DUMP;
   // bring the carry back to the exact maximum
   {
     const float m_safe = (m_true == RA_NEG_INF) ? 0.f : m_true;
