@@ -10,7 +10,13 @@
 //    64-key tiles of K and V through LDS.  Scores are produced transposed (S^T = K Q^T),
 //    exactly as in the forward kernel, so dS^T is the B operand of dQ^T = K^T dS^T.
 // Plus the elementwise delta = rowsum(out * dout) and the fp32 -> bf16 gradient cast.
+#include <type_traits>
+
 #include "ra_launch.h"
+
+#ifndef RA_ABLATE_B
+#define RA_ABLATE_B 0  // timing experiments only: bit mask of loop parts to leave out
+#endif
 
 namespace ra {
 
@@ -49,25 +55,35 @@ __global__ void bwd_delta_kernel(const OutT* out, long long sb, long long sh, lo
 // ------------------------------------------------------------------------------------------------
 constexpr int kQTile = 32;  // queries per LDS tile in dkdv_kernel
 
-template <int D, int NKB, bool GENERAL>
+// One workgroup = 4 waves = 128 keys; every wave owns 32 keys for the whole kernel: their K
+// and V rows sit in registers as MFMA B operands and the 32 x D dK and dV accumulators in
+// accumulation registers (one wave per SIMD, 512 registers).  32-query tiles of Q and dO are
+// streamed through three LDS buffers with direct-to-LDS loads.  Inside a wave the matrix unit
+// runs one tile ahead of the vector ALU: the 16 MFMAs of S(i+1) = Q K^T and dP(i+1) = dO V^T
+// carry, in their shadow, the exp2 / dS arithmetic of tile i; then come the 16 MFMAs of
+// dV += P(i)^T dO and dK += dS(i)^T Q.
+template <int D, bool GENERAL>
 __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   constexpr int NT = 256;
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
-  constexpr int KEYS_WG = 4 * 32 * NKB;
-  constexpr int TILE_BYTES = kQTile * D * 2;
+  constexpr int KEYS_WG = 128;
+  constexpr int ROWB = D * 2;
+  constexpr int TILE_BYTES = kQTile * ROWB;
 
-  __shared__ __attribute__((aligned(16))) char s_q[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char s_do[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) float s_lse[2][kQTile];
-  __shared__ __attribute__((aligned(16))) float s_delta[2][kQTile];
-  __shared__ __attribute__((aligned(16))) int s_seg[2][kQTile];
-  __shared__ __attribute__((aligned(16))) int s_pre[2][kQTile];
+  __shared__ __attribute__((aligned(16))) char s_q[3][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char s_do[3][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) float s_lse[3][kQTile];
+  __shared__ __attribute__((aligned(16))) float s_delta[3][kQTile];
+  __shared__ __attribute__((aligned(16))) int s_seg[3][kQTile];
+  __shared__ __attribute__((aligned(16))) int s_pre[3][kQTile];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[12];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
   const int nkt = (a.Lk + KEYS_WG - 1) / KEYS_WG;
   int hh, kt;
@@ -75,32 +91,32 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   kt = nkt - 1 - kt;  // under a causal mask the FIRST key slab has the most work
   const int b = hh / a.H, h = hh % a.H;
   const int k0 = kt * KEYS_WG;
-  const int kw = k0 + wave * 32 * NKB;
+  const int kw = k0 + wave * 32;
   const BiasArgs& bs = a.bias;
   const int flags = bs.flags;
+  const bool wave_on = kw < a.Lk;
 
   // ---- resident key-side operands ----------------------------------------------------------
-  bf16x8 kf[NKB][KS], vf[NKB][KS];
-  int k_seg[NKB], k_pre[NKB];
-#pragma unroll
-  for (int kb = 0; kb < NKB; ++kb) {
-    const int ki = min(kw + 32 * kb + l32, a.Lk - 1);
+  bf16x8 kf[KS], vf[KS];
+  int k_seg = 0, k_pre = 0;
+  {
+    const int ki = min(kw + l32, a.Lk - 1);
     const bf16_t* kp = a.k.ptr + b * a.k.sb + h * a.k.sh + (long long)ki * a.k.sl + 8 * g;
     const bf16_t* vp = a.v.ptr + b * a.v.sb + h * a.v.sh + (long long)ki * a.v.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      kf[kb][s] = *(const bf16x8*)(kp + 16 * s);
-      vf[kb][s] = *(const bf16x8*)(vp + 16 * s);
+      kf[s] = *(const bf16x8*)(kp + 16 * s);
+      vf[s] = *(const bf16x8*)(vp + 16 * s);
     }
-    k_seg[kb] = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.kv_seg[b * bs.kv_seg_sb + ki] : 0;
-    k_pre[kb] = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.kv_pre[b * bs.kv_pre_sb + ki] : 0;
+    if (GENERAL && (flags & RA_BIAS_SEGMENT)) k_seg = bs.kv_seg[b * bs.kv_seg_sb + ki];
+    if (GENERAL && (flags & RA_BIAS_PREFIX)) k_pre = bs.kv_pre[b * bs.kv_pre_sb + ki];
   }
   float slope2 = 0.f;
   if (GENERAL && (flags & RA_BIAS_ALIBI)) slope2 = bs.slopes[h] * kLog2e;
   const int* q_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.q_seg + b * bs.q_seg_sb : nullptr;
   const int* q_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.q_pre + b * bs.q_pre_sb : nullptr;
 
-  f32x16 dk[NKB][DB], dv[NKB][DB];
+  f32x16 dk[DB], dv[DB];
   {
     // zero the accumulators THROUGH the matrix unit so that they are born in accumulation
     // registers and stay there for the whole loop
@@ -111,12 +127,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) z16[r] = 0.f;
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        dk[kb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
-        dv[kb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
-      }
+    for (int db = 0; db < DB; ++db) {
+      dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
+      dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
+    }
   }
 
   // ---- which query tiles does this workgroup visit -------------------------------------------
@@ -129,12 +143,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     use_list = true;
     int smin = 0x7fffffff, smax = (int)0x80000000;
-#pragma unroll
-    for (int kb = 0; kb < NKB; ++kb)
-      if (kw + 32 * kb + l32 < a.Lk) {
-        smin = min(smin, k_seg[kb]);
-        smax = max(smax, k_seg[kb]);
-      }
+    if (kw + l32 < a.Lk) {
+      smin = k_seg;
+      smax = k_seg;
+    }
     smin = wave_min(smin);
     smax = wave_max(smax);
     if (lane == 0) {
@@ -175,14 +187,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     __syncthreads();
     n_act = s_red[8];
   }
-
-  const bf16_t* qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
-  const bf16_t* dobase = a.dout.ptr + b * a.dout.sb + h * a.dout.sh;
-  const float* lse_row = a.lse + ((long long)b * a.H + h) * a.Lq;
-  const float* delta_row = a.delta + ((long long)b * a.H + h) * a.Lq;
-  TileStage<D, kQTile, NT> qst, dost;
-  float lse_r = 0.f, delta_r = 0.f;
-  int seg_r = 0, pre_r = 0;
+  const int n = n_act;
 
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
@@ -193,127 +198,301 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     segbit = 0;
     return i_lo + i;
   };
-  auto issue_loads = [&](int it) {
-    qst.load(qbase, a.q.sl, it * kQTile, a.Lq, tid);
-    dost.load(dobase, a.dout.sl, it * kQTile, a.Lq, tid);
-    if (tid < kQTile) {
-      const int qq = min(it * kQTile + tid, a.Lq - 1);
-      const float L = lse_row[qq];
-      lse_r = (L == RA_NEG_INF) ? __builtin_inff() : L * kLog2e;  // fully masked row: P = 0
+
+  // ---- global -> LDS ---------------------------------------------------------------------------
+  // every wave moves 8 of a tile's 32 rows of Q and of dO; lane l of a load instruction fills
+  // physical chunk l % CPR of row l / CPR and fetches the logical chunk the XOR layout puts there
+  const bf16_t* qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
+  const bf16_t* dobase = a.dout.ptr + b * a.dout.sb + h * a.dout.sh;
+  const float* lse_row = a.lse + ((long long)b * a.H + h) * a.Lq;
+  const float* delta_row = a.delta + ((long long)b * a.H + h) * a.Lq;
+  constexpr int CPR = D / 8;
+  constexpr int RPI = 64 / CPR;
+  constexpr int NLD = 8 / RPI;
+  int ld_row[NLD], ld_off[NLD];
+  unsigned q_voff[NLD], do_voff[NLD];  // per-lane byte offsets inside a group of RPI rows
+#pragma unroll
+  for (int t = 0; t < NLD; ++t) {
+    const int rrow = 8 * wave + RPI * t + lane / CPR;
+    const int pc = lane % CPR;
+    ld_row[t] = rrow;
+    ld_off[t] = ((tile_off<D>(rrow, pc) - rrow * ROWB) >> 4) * 8;
+    q_voff[t] = (unsigned)(((long long)(lane / CPR) * a.q.sl + ld_off[t]) * 2);
+    do_voff[t] = (unsigned)(((long long)(lane / CPR) * a.dout.sl + ld_off[t]) * 2);
+  }
+  float lse_r = 0.f, delta_r = 0.f;
+  int seg_r = 0, pre_r = 0;
+  auto issue_tile = [&](int it, int buf) {
+    const int q0 = it * kQTile;
+    const unsigned q_dst = RA_LDS_ADDR(&s_q[0][0]) + buf * TILE_BYTES + wave_u * 8 * ROWB;
+    const unsigned do_dst = RA_LDS_ADDR(&s_do[0][0]) + buf * TILE_BYTES + wave_u * 8 * ROWB;
+    if (RA_ABLATE_B & 1) {
+    } else if (q0 + kQTile <= a.Lq) {
+      // wave-uniform row addresses in scalar registers, per-lane part in one VGPR
+      const bf16_t* qs = qbase + (long long)(q0 + 8 * wave_u) * a.q.sl;
+      const bf16_t* ds = dobase + (long long)(q0 + 8 * wave_u) * a.dout.sl;
+      if (NLD == 2) {
+        global_to_lds16_s_x2(qs, q_voff[0], qs + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1], q_dst);
+        global_to_lds16_s_x2(ds, do_voff[0], ds + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1], do_dst);
+      } else {
+        global_to_lds16_s(qs, q_voff[0], q_dst);
+        global_to_lds16_s(ds, do_voff[0], do_dst);
+      }
+    } else {  // last, partial tile: rows past the end repeat the last row (masked later)
+#pragma unroll
+      for (int t = 0; t < NLD; ++t) {
+        const int gr = min(q0 + ld_row[t], a.Lq - 1);
+        global_to_lds16(qbase + (long long)gr * a.q.sl + ld_off[t], q_dst + RPI * t * ROWB);
+        global_to_lds16(dobase + (long long)gr * a.dout.sl + ld_off[t], do_dst + RPI * t * ROWB);
+      }
+    }
+    if (tid < kQTile && !(RA_ABLATE_B & 2)) {  // values are consumed in store_rows, one iteration later
+      const int qq = min(q0 + tid, a.Lq - 1);
+      lse_r = lse_row[qq];
       delta_r = delta_row[qq];
       if (GENERAL && q_seg) seg_r = q_seg[qq];
       if (GENERAL && q_pre) pre_r = q_pre[qq];
     }
   };
-
-  int sb0 = 0;
-  if (n_act > 0) issue_loads(tile_at(0, sb0));
-
-  for (int i = 0; i < n_act; ++i) {
-    const int buf = i & 1;
-    qst.store(s_q[buf], tid);
-    dost.store(s_do[buf], tid);
+  auto store_rows = [&](int buf) {
     if (tid < kQTile) {
-      s_lse[buf][tid] = lse_r;
+      // log2 domain; a fully masked row (lse = -inf) becomes +inf so that its P is 0
+      s_lse[buf][tid] = (lse_r == RA_NEG_INF) ? __builtin_inff() : lse_r * kLog2e;
       s_delta[buf][tid] = delta_r;
       if (GENERAL) {
         s_seg[buf][tid] = seg_r;
         s_pre[buf][tid] = pre_r;
       }
     }
-    __syncthreads();
-    int cur_segbit;
-    const int it = tile_at(i, cur_segbit);
-    if (i + 1 < n_act) {
-      int nb;
-      issue_loads(tile_at(i + 1, nb));
+  };
+
+  // per-lane LDS offsets of the operand fetches (the tile buffer and the 16-row step fold into
+  // the instructions' immediate offsets)
+  int noff[KS];
+#pragma unroll
+  for (int ss = 0; ss < KS; ++ss) noff[ss] = tile_off<D>(l32, 2 * ss + g);
+  int toff[DB][2];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int j = lane & 15;
+      const int trow = 4 * g + (j >> 2) + 8 * h2;
+      const int tcol = 32 * db + 16 * ((lane >> 4) & 1) + 4 * (j & 3);
+      toff[db][h2] = tile_off<D>(trow, tcol >> 3) + ((tcol & 4) << 1);
     }
-    const int qt0 = it * kQTile;
-    const int qlo = bs.q_off + qt0, qhi = qlo + kQTile - 1;
-    const bool ragged = qt0 + kQTile > a.Lq;
+  auto nat_frag = [&](const char* tile, int ss) { return *(const bf16x8*)(tile + noff[ss]); };
+  auto tr_frag = [&](const char* tile, int ks, int db) {
+    const lds_char* p0 = (const lds_char*)(tile + 16 * ks * ROWB + toff[db][0]);
+    const lds_char* p1 = (const lds_char*)(tile + 16 * ks * ROWB + toff[db][1]);
+    bf16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p0);
+    bf16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p1);
+    return __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
 
+  // positional class of this wave's 32 keys against query tile index i
+  auto tile_class = [&](int i, int& qt0, int& segbit) -> int {
+    qt0 = tile_at(i, segbit) * kQTile;
+    if (flags & RA_BIAS_PREFIX) return 2;
+    return classify_pos(flags, bs.window, bs.q_off + qt0, bs.q_off + qt0 + kQTile - 1, bs.kv_off + kw,
+                        bs.kv_off + kw + 31);
+  };
+  auto needs_bias = [&](int qt0, int segbit, int cls) -> bool {
+    bool nb = (cls & 2) || (qt0 + kQTile > a.Lq);
+    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
+    return nb;
+  };
+  // S = Q K^T and dP = dO V^T of one tile, nothing interleaved
+  constexpr int PF = 3;
+  auto compute_s_dp = [&](f32x16& S, f32x16& P, const char* qt, const char* dot) {
+    bf16x8 fr[2 * KS];
 #pragma unroll
-    for (int kb = 0; kb < NKB; ++kb) {
-      const int kb0 = kw + 32 * kb;
-      if (kb0 >= a.Lk) continue;
-      const int klo = bs.kv_off + kb0, khi = klo + 31;
-      const int cls = (flags & RA_BIAS_PREFIX) ? 2 : classify_pos(flags, bs.window, qlo, qhi, klo, khi);
-      if (cls & 1) continue;
-      TileBias tb;
-      tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
-      if (GENERAL) {
-        tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
-        if (cur_segbit) tb.flags |= RA_BIAS_SEGMENT;
+    for (int r = 0; r < 16; ++r) {
+      S[r] = 0.f;
+      P[r] = 0.f;
+    }
+#pragma unroll
+    for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? dot : qt, op >> 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 2 * KS; ++op) {
+      if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? dot : qt, (op + PF) >> 1);
+      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], P, 0, 0, 0);
+      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], S, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // dV += P^T dO and dK += dS^T Q of one tile
+  auto compute_dkdv = [&](const bf16x8 (&pf)[2], const bf16x8 (&dsf)[2], const char* qt, const char* dot) {
+    bf16x8 fr[4 * DB];
+#pragma unroll
+    for (int op = 0; op < PF; ++op) fr[op] = tr_frag((op & 1) ? qt : dot, op / (2 * DB), (op >> 1) % DB);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 4 * DB; ++op) {
+      if (op + PF < 4 * DB) {
+        const int o2 = op + PF;
+        fr[o2] = tr_frag((o2 & 1) ? qt : dot, o2 / (2 * DB), (o2 >> 1) % DB);
       }
-      tb.window = bs.window;
-      tb.slope2 = slope2;
-      tb.var_limit = a.Lq - (qt0 + 4 * g);
+      const int ks = op / (2 * DB), db = (op >> 1) % DB;
+      if (op & 1) dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[ks], fr[op], dk[db], 0, 0, 0);
+      else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], fr[op], dv[db], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // scale + bias of a fresh S in place (rows of the accumulator are queries)
+  auto prepare = [&](f32x16& S, int qt0, int segbit, int cls, int ids_buf) {
+    TileBias tb;
+    tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
+    if (GENERAL) {
+      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
+      if (segbit) tb.flags |= RA_BIAS_SEGMENT;
+    }
+    tb.window = bs.window;
+    tb.slope2 = slope2;
+    tb.var_limit = a.Lq - (qt0 + 4 * g);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] *= a.scale2;
+    const int rel0 = (bs.q_off + qt0 + 4 * g) - (bs.kv_off + kw + l32);
+    apply_bias<false>(S, tb, rel0, k_seg, k_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
+  };
 
-      // S = Q K^T and dP = dO V^T for 32 queries x 32 keys
-      f32x16 sacc, pacc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        sacc[r] = 0.f;
-        pacc[r] = 0.f;
-      }
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        bf16x8 qa = frag_nat<D>(s_q[buf], l32, s, g);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kb][s], sacc, 0, 0, 0);
-      }
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        bf16x8 da = frag_nat<D>(s_do[buf], l32, s, g);
-        pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[kb][s], pacc, 0, 0, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[r] *= a.scale2;
-      if (tb.flags != 0 || ragged) {
-        const int rel0 = (bs.q_off + qt0 + 4 * g) - (bs.kv_off + kb0 + l32);
-        apply_bias<false>(sacc, tb, rel0, k_seg[kb], k_pre[kb], &s_seg[buf][4 * g], &s_pre[buf][4 * g]);
-      }
-      // P = exp2(t - lse2), dS = P * (dP - delta); rows of the accumulator are queries
-#pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        const f32x4 L4 = *(const f32x4*)&s_lse[buf][8 * bb + 4 * g];
-        const f32x4 d4 = *(const f32x4*)&s_delta[buf][8 * bb + 4 * g];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          const int r = 4 * bb + c;
-          const float p = fast_exp2(sacc[r] - L4[c]);
-          sacc[r] = p;
-          pacc[r] = p * (pacc[r] - d4[c]);
-        }
-      }
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const bf16x8 pf = pack8(sacc, 8 * ks);
-        const bf16x8 dsf = pack8(pacc, 8 * ks);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          bf16x8 dob = frag_tr<D>(s_do[buf], 16 * ks, 32 * db, lane);
-          dv[kb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf, dob, dv[kb][db], 0, 0, 0);
-          bf16x8 qb = frag_tr<D>(s_q[buf], 16 * ks, 32 * db, lane);
-          dk[kb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf, qb, dk[kb][db], 0, 0, 0);
-        }
-      }
+  // ---- prologue: tiles 0 and 1 in flight, S(0) and dP(0) computed -----------------------------
+  if (n > 0) {
+    int sbu;
+    issue_tile(tile_at(0, sbu), 0);
+    store_rows(0);
+  }
+  if (n > 1) {
+    int sbu;
+    issue_tile(tile_at(1, sbu), 1);  // its rows are stored at the top of iteration 0
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+
+  f32x16 s_a, p_a, s_b, p_b, s_c, p_c;
+  bool cur_valid = false, cur_scaled = false;
+  if (n > 0 && wave_on) {
+    int qt0, segbit;
+    const int cls = tile_class(0, qt0, segbit);
+    if (!(cls & 1)) {
+      cur_valid = true;
+      compute_s_dp(s_a, p_a, s_q[0], s_do[0]);
+      cur_scaled = needs_bias(qt0, segbit, cls);
+      if (cur_scaled) prepare(s_a, qt0, segbit, cls, 0);
     }
   }
 
+  RA_PROF_DECL
+  // one iteration; (SC, PC) hold S(i), dP(i) on entry, (SN, PN) receive S(i+1), dP(i+1).
+  // Tile j lives in LDS buffer j % 3 = PH for j = i.
+  auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
+    constexpr int PH = decltype(phase)::value;
+    constexpr int PH1 = (PH + 1) % 3, PH2 = (PH + 2) % 3;
+    RA_PROF_MARK(i, 1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+1 is in LDS
+    if (i + 1 < n) store_rows(PH1);      // its per-row lse / delta / ids arrived with it
+    __syncthreads();
+    RA_PROF_MARK(i, 2);
+    if (i + 2 < n) {
+      int sbu;
+      issue_tile(tile_at(i + 2, sbu), PH2);
+    }
+    const char* qc = s_q[PH];
+    const char* doc = s_do[PH];
+    const char* qn = s_q[PH1];
+    const char* don = s_do[PH1];
+    int nqt0 = 0, nsegbit = 0, ncls = 1;
+    bool nxt_valid = false;
+    if (i + 1 < n && wave_on) {
+      ncls = tile_class(i + 1, nqt0, nsegbit);
+      nxt_valid = !(ncls & 1);
+    }
+    const bool nxt_scaled = nxt_valid && needs_bias(nqt0, nsegbit, ncls);
+    bf16x8 pf[2], dsf[2];
+    // per-row statistics of tile i: this lane's 16 query rows are 8*bb + 4*g + c
+    f32x4 L4[4], D4[4];
+    if (cur_valid) {
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        L4[bb] = *(const f32x4*)&s_lse[PH][8 * bb + 4 * g];
+        D4[bb] = *(const f32x4*)&s_delta[PH][8 * bb + 4 * g];
+      }
+    }
+    RA_PROF_MARK(i, 3);
+    if (cur_valid && nxt_valid && !cur_scaled) {
+      // ---- fused: S(i+1), dP(i+1) MFMAs with P(i), dS(i) arithmetic in their shadow -------------
+      bf16x8 fr[2 * KS];
+#pragma unroll
+      for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? don : qn, op >> 1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int op = 0; op < 2 * KS; ++op) {
+        if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? don : qn, (op + PF) >> 1);
+        if (op < 2) {
+          // first link of each chain starts from a zero accumulator
+          f32x16 z;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) z[r] = 0.f;
+          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], z, 0, 0, 0);
+          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], z, 0, 0, 0);
+        } else {
+          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], PN, 0, 0, 0);
+          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], SN, 0, 0, 0);
+        }
+        constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+        if (op * EPO < 16) {
+#pragma unroll
+          for (int e = 0; e < EPO; ++e) {
+            const int r = op * EPO + e;
+            const float p = fast_exp2(fmaf(SC[r], a.scale2, -L4[r >> 2][r & 3]));
+            const float ds = p * (PC[r] - D4[r >> 2][r & 3]);
+            pf[r >> 3][r & 7] = (bf16_t)p;
+            dsf[r >> 3][r & 7] = (bf16_t)ds;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      RA_PROF_MARK(i, 4);
+      compute_dkdv(pf, dsf, qc, doc);
+      RA_PROF_MARK(i, 5);
+    } else {
+      if (nxt_valid) compute_s_dp(SN, PN, qn, don);
+      if (cur_valid) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float t = cur_scaled ? SC[r] - L4[r >> 2][r & 3] : fmaf(SC[r], a.scale2, -L4[r >> 2][r & 3]);
+          const float p = fast_exp2(t);
+          const float ds = p * (PC[r] - D4[r >> 2][r & 3]);
+          pf[r >> 3][r & 7] = (bf16_t)p;
+          dsf[r >> 3][r & 7] = (bf16_t)ds;
+        }
+        compute_dkdv(pf, dsf, qc, doc);
+      }
+    }
+    if (nxt_scaled) prepare(SN, nqt0, nsegbit, ncls, PH1);
+    cur_valid = nxt_valid;
+    cur_scaled = nxt_scaled;
+    RA_PROF_MARK(i, 6);
+  };
+
+  for (int i = 0; i < n; i += 3) {
+    iteration(std::integral_constant<int, 0>{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(std::integral_constant<int, 1>{}, i + 1, s_b, p_b, s_c, p_c);
+    if (i + 2 < n) iteration(std::integral_constant<int, 2>{}, i + 2, s_c, p_c, s_a, p_a);
+  }
+
+  RA_PROF_DUMP;
   // ---- accumulate into the fp32 gradients owned by this key slab ------------------------------
 #pragma unroll
-  for (int kb = 0; kb < NKB; ++kb) {
-    const int kb0 = kw + 32 * kb;
+  for (int r = 0; r < 16; ++r) {
+    const int key = kw + 8 * (r / 4) + 4 * g + (r % 4);
+    if (key < a.Lk) {
+      const long long off = (((long long)b * a.H + h) * a.Lk + key) * D + l32;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int key = kb0 + 8 * (r / 4) + 4 * g + (r % 4);
-      if (key < a.Lk) {
-        const long long off = (((long long)b * a.H + h) * a.Lk + key) * D + l32;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          a.dk[off + 32 * db] += dk[kb][db][r] * a.sm_scale;
-          a.dv[off + 32 * db] += dv[kb][db][r];
-        }
+      for (int db = 0; db < DB; ++db) {
+        a.dk[off + 32 * db] += dk[db][r] * a.sm_scale;
+        a.dv[off + 32 * db] += dv[db][r];
       }
     }
   }
@@ -593,19 +772,17 @@ hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long lon
   return hipGetLastError();
 }
 
-constexpr int kNkb = 1;  // 32-key blocks per wave in dkdv_kernel
-
 hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, int parts, hipStream_t stream) {
   if (parts & 1) {
-    const int keys_wg = 4 * 32 * kNkb;
+    const int keys_wg = 128;
     const int nkt = (a.Lk + keys_wg - 1) / keys_wg;
     dim3 grid((unsigned)(a.B * a.H * nkt)), block(256);
     if (D == 128) {
-      if (general) hipLaunchKernelGGL((dkdv_kernel<128, kNkb, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dkdv_kernel<128, kNkb, false>), grid, block, 0, stream, a);
+      if (general) hipLaunchKernelGGL((dkdv_kernel<128, true>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((dkdv_kernel<128, false>), grid, block, 0, stream, a);
     } else {
-      if (general) hipLaunchKernelGGL((dkdv_kernel<64, kNkb, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dkdv_kernel<64, kNkb, false>), grid, block, 0, stream, a);
+      if (general) hipLaunchKernelGGL((dkdv_kernel<64, true>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((dkdv_kernel<64, false>), grid, block, 0, stream, a);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;

@@ -12,6 +12,7 @@ namespace ra {
 typedef __bf16 bf16_t;
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
@@ -169,14 +170,27 @@ struct TileStage {
   }
 };
 
-// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_base + 16*l
-// (lds_base is wave-uniform and goes through M0).  Issued as inline assembly so that the
-// compiler does not guard later, unrelated LDS reads with a full vmcnt wait; completion is
-// the caller's business (s_waitcnt vmcnt(0) before the barrier that publishes the tile).
-RA_DEV void global_to_lds16(const void* gptr, const char* lds_base) {
-  const unsigned lds_addr = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(const lds_char*)lds_base);
+// 16 bytes per lane from global memory straight into LDS: lane l lands at lds_addr + 16*l.
+// lds_addr is a wave-uniform LDS byte address (it travels through M0).  The global address is
+// a wave-uniform 64-bit base (scalar registers) plus a per-lane unsigned 32-bit byte offset.
+// Issued as inline assembly so that the compiler does not guard later, unrelated LDS reads
+// with a full vmcnt wait; completion is the caller's business (s_waitcnt vmcnt(0) before the
+// barrier that publishes the tile).  The "x2" form moves two pieces that are 1 KiB apart in
+// LDS with one M0 write: the instruction offset applies to the LDS address AND to the global
+// address, so the second base must already have 1024 bytes subtracted.
+RA_DEV void global_to_lds16(const void* gptr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
+RA_DEV void global_to_lds16_s(const void* sbase, unsigned voff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory", "m0");
+}
+RA_DEV void global_to_lds16_s_x2(const void* sbase0, unsigned voff0, const void* sbase1_minus_1k, unsigned voff1,
+                                 unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %4\n\tglobal_load_lds_dwordx4 %1, %0\n\tglobal_load_lds_dwordx4 %3, %2 offset:1024"
+               : : "s"(sbase0), "v"(voff0), "s"(sbase1_minus_1k), "v"(voff1), "s"(lds_addr) : "memory", "m0");
+}
+// LDS byte address of an object declared __shared__
+#define RA_LDS_ADDR(obj) ((unsigned)(uintptr_t)(lds_char*)(obj))
 
 RA_DEV bf16x8 pack8(const f32x16& p, int base) {
   bf16x8 r;

@@ -37,7 +37,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
   __shared__ int s_red[20];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   int hh, qt;
@@ -59,20 +61,24 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
   }
   const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
-  float m_run = a.m[row] * kLog2e;
-  float l_run = (g == 0) ? a.l[row] : 0.f;
+  // This step accumulates its own contribution from zero and is merged with the incoming carry
+  // at the end.  Two row sums are kept: l_run adds the fp32 probabilities (it becomes the
+  // carry's l and the logsumexp), lr_run adds the SAME probabilities after their rounding to
+  // bf16, i.e. the weights that actually multiply V.  Scaling the step's output by
+  // l_run / lr_run makes it a properly normalised average of V times the exact row sum, so
+  // the rounding of P cancels in o / l instead of showing up as an error of order 2^-9 |v|
+  // on rows that see only a few keys.
+  const float m_in = a.m[row] * kLog2e;
+  float m_run = m_in;  // exponent reference (log2 domain), moves lazily
+  float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
   f32x16 oacc[DB];
-  {
-    const float* op = a.o + row * D + 4 * g;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        f32x4 t = *(const f32x4*)(op + 32 * db + 8 * bb);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) oacc[db][4 * bb + c] = t[c];
-      }
-  }
+    for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
+  bf16x2 ones2;
+  ones2[0] = (bf16_t)1.0f;
+  ones2[1] = (bf16_t)1.0f;
   int q_seg = 0, q_pre = 0;
   float slope2 = 0.f;
   if (GENERAL) {
@@ -159,6 +165,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   constexpr int RPI = 64 / CPR;         // rows per load instruction
   constexpr int NLD = 8 / RPI;          // load instructions per wave per tile
   int ld_row[NLD], ld_koff[NLD];
+  unsigned k_voff[NLD], v_voff[NLD];  // per-lane byte offsets inside a group of RPI rows
 #pragma unroll
   for (int t = 0; t < NLD; ++t) {
     const int rrow = 8 * wave + RPI * t + lane / CPR;
@@ -166,15 +173,25 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     const int lc = (tile_off<D>(rrow, pc) - rrow * (D * 2)) >> 4;  // logical chunk stored at pc
     ld_row[t] = rrow;
     ld_koff[t] = lc * 8;
+    k_voff[t] = (unsigned)(((long long)(lane / CPR) * a.k.sl + lc * 8) * 2);
+    v_voff[t] = (unsigned)(((long long)(lane / CPR) * a.v.sl + lc * 8) * 2);
   }
+  auto issue_rows = [&](const bf16_t* base, const unsigned (&voff)[NLD], long long sl, int k0, unsigned dst) {
+    if (k0 + kKeyTile <= a.Lk) {
+      const bf16_t* sb = base + (long long)(k0 + 8 * wave_u) * sl;  // wave-uniform: scalar registers
+      if (NLD == 2) global_to_lds16_s_x2(sb, voff[0], sb + (long long)RPI * sl - 512, voff[NLD - 1], dst);
+      else global_to_lds16_s(sb, voff[0], dst);
+    } else {  // last, partial tile: rows past the end repeat the last row (masked later)
+#pragma unroll
+      for (int t = 0; t < NLD; ++t) {
+        const int gr = min(k0 + ld_row[t], a.Lk - 1);
+        global_to_lds16(base + (long long)gr * sl + ld_koff[t], dst + RPI * t * (D * 2));
+      }
+    }
+  };
   auto issue_k = [&](int j, int buf) {
     const int k0 = j * kKeyTile;
-#pragma unroll
-    for (int t = 0; t < NLD; ++t) {
-      const int gr = min(k0 + ld_row[t], a.Lk - 1);
-      const bf16_t* src = kbase + (long long)gr * a.k.sl + ld_koff[t];
-      global_to_lds16(src, s_k[buf] + (8 * wave + RPI * t) * (D * 2));
-    }
+    issue_rows(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + buf * TILE_BYTES + wave_u * 8 * (D * 2));
     if (GENERAL && tid < kKeyTile) {
       int kk = min(k0 + tid, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
@@ -182,13 +199,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     }
   };
   auto issue_v = [&](int j, int buf) {
-    const int k0 = j * kKeyTile;
-#pragma unroll
-    for (int t = 0; t < NLD; ++t) {
-      const int gr = min(k0 + ld_row[t], a.Lk - 1);
-      const bf16_t* src = vbase + (long long)gr * a.v.sl + ld_koff[t];
-      global_to_lds16(src, s_v[buf] + (8 * wave + RPI * t) * (D * 2));
-    }
+    issue_rows(vbase, v_voff, a.v.sl, j * kKeyTile, RA_LDS_ADDR(&s_v[0][0]) + buf * TILE_BYTES + wave_u * 8 * (D * 2));
   };
   const int n = n_act;
   int sb_unused;
@@ -341,6 +352,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       const float corr = fast_exp2(m_run - m_safe_new);
       m_run = m_new;
       l_run *= corr;
+      lr_run *= corr;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -416,8 +428,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
             const float p1 = fast_exp2(fmaf(SC[kb][r + 1], a.scale2, neg_m));
             rs0 += p0;
             rs1 += p1;
-            pfrag[2 * kb + (r >> 3)][r & 7] = (bf16_t)p0;
-            pfrag[2 * kb + (r >> 3)][(r & 7) + 1] = (bf16_t)p1;
+            bf16x2 pr;
+            pr[0] = (bf16_t)p0;
+            pr[1] = (bf16_t)p1;
+            lr_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lr_run, false);
+            pfrag[2 * kb + (r >> 3)][r & 7] = pr[0];
+            pfrag[2 * kb + (r >> 3)][(r & 7) + 1] = pr[1];
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -465,7 +481,16 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-          for (int ks = 0; ks < 2; ++ks) pfrag[2 * kb + ks] = pack8(SC[kb], 8 * ks);
+          for (int ks = 0; ks < 2; ++ks) {
+            pfrag[2 * kb + ks] = pack8(SC[kb], 8 * ks);
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+              bf16x2 pr;
+              pr[0] = pfrag[2 * kb + ks][e];
+              pr[1] = pfrag[2 * kb + ks][e + 1];
+              lr_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lr_run, false);
+            }
+          }
         compute_pv(pfrag, vt);
       }
       if (nxt_valid && !nxt_scaled) nxt_mx = raw_rowmax(SN);
@@ -484,36 +509,33 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   }
 
   RA_PROF_DUMP;
-  // bring the carry back to the exact maximum
+  // ---- merge this step into the carry ---------------------------------------------------------
+  // o = o_in 2^(m_in - m_out) + o_step 2^(m_run - m_out) l_step / lr_step,  l likewise with the
+  // exact sum, m_out = exact maximum over carry and step.
   {
-    const float m_safe = (m_true == RA_NEG_INF) ? 0.f : m_true;
-    const float f = fast_exp2(m_run - m_safe);  // 1 where the reference is exact, 0 for empty rows
-    if (__any(m_run != m_true)) {
-      l_run *= f;
+    const float l_step = half_sum(l_run), lr_step = half_sum(lr_run);
+    const float m_out = m_true;  // started from m_in, so it already covers the carry
+    const float m_safe = (m_out == RA_NEG_INF) ? 0.f : m_out;
+    const float f_in = fast_exp2(m_in - m_safe);   // 0 for an empty carry
+    float f_step = fast_exp2(m_run - m_safe);      // 1 where the reference is exact
+    const float ratio = (lr_step > 0.f) ? l_step / lr_step : 1.f;
+    const float l_out = a.l[row] * f_in + l_step * f_step;
+    f_step *= ratio;
+    if (q_valid) {
+      float* op = a.o + row * D + 4 * g;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] *= f;
-    }
-    m_run = m_true;
-  }
-
-  // ---- write the carry back ------------------------------------------------------------------
-  const float l_tot = half_sum(l_run);
-  if (q_valid) {
-    float* op = a.o + row * D + 4 * g;
+        for (int bb = 0; bb < 4; ++bb) {
+          f32x4 t = *(const f32x4*)(op + 32 * db + 8 * bb);
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        f32x4 t;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) t[c] = oacc[db][4 * bb + c];
-        *(f32x4*)(op + 32 * db + 8 * bb) = t;
+          for (int c = 0; c < 4; ++c) t[c] = t[c] * f_in + oacc[db][4 * bb + c] * f_step;
+          *(f32x4*)(op + 32 * db + 8 * bb) = t;
+        }
+      if (g == 0) {
+        a.m[row] = m_out * kLn2;
+        a.l[row] = l_out;
       }
-    if (g == 0) {
-      a.m[row] = m_run * kLn2;
-      a.l[row] = l_tot;
     }
   }
 }
