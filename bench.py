@@ -87,7 +87,7 @@ class EventTimer:
 
 def cpu_baseline(D):
     """The numpy restatement of the reference algorithm, timed on the host cores on a bounded
-    sample of the workload (same head dim, causal, fp32): H=2, S=8192 as 2 shards of 4096."""
+    sample of the workload (same head dim, causal, fp32): H=8, S=16384 as 4 shards of 4096."""
     import numpy as np
     from oracle import ring_oracle as R
     try:
@@ -95,7 +95,7 @@ def cpu_baseline(D):
         threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
     except Exception:
         threads = os.cpu_count() or 1
-    H, S, n = 2, 8192, 2
+    H, S, n = 8, 16384, 4
     q, k, v, do = R.make_inputs(0, 1, S, S, H, D)
     pos = np.broadcast_to(np.arange(S), (1, S))
     fn = R.make_bias_fn(causal=True)
