@@ -370,6 +370,17 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
+  // Ordinals [plain_lo, plain_hi) of the query tiles this wave's keys see completely, unmasked
+  // and in range: they take the fused path without any per-tile classification.
+  int plain_lo = 0, plain_hi = 0;
+  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT)))) {
+    int lo, hi;
+    query_tile_plain_range(flags, bs.window, bs.kv_off + kw, bs.kv_off + kw + 31, bs.q_off, a.Lq / kQTile,
+                           kQTile, lo, hi);
+    plain_lo = max(lo - i_lo, 0);
+    plain_hi = min(hi - i_lo, n);
+  }
+
   f32x16 s_a, p_a, s_b, p_b, s_c, p_c;
   bool cur_valid = false, cur_scaled = false;
   if (n > 0 && wave_on) {
@@ -403,12 +414,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     const char* qn = s_q[PH1];
     const char* don = s_do[PH1];
     int nqt0 = 0, nsegbit = 0, ncls = 1;
-    bool nxt_valid = false;
-    if (i + 1 < n && wave_on) {
+    bool nxt_valid = false, nxt_scaled = false;
+    if (i + 1 >= plain_lo && i + 1 < plain_hi) {
+      nxt_valid = true;
+    } else if (i + 1 < n && wave_on) {
       ncls = tile_class(i + 1, nqt0, nsegbit);
       nxt_valid = !(ncls & 1);
+      nxt_scaled = nxt_valid && needs_bias(nqt0, nsegbit, ncls);
     }
-    const bool nxt_scaled = nxt_valid && needs_bias(nqt0, nsegbit, ncls);
     bf16x8 pf[2], dsf[2];
     // per-row statistics of tile i: this lane's 16 query rows are 8*bb + 4*g + c
     f32x4 L4[4], D4[4];
@@ -502,24 +515,36 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 // dQ
 // ------------------------------------------------------------------------------------------------
 constexpr int kDqThreads = 512;
-constexpr int kDqRows = 256;
-constexpr int kDqKeyTile = 64;
+constexpr int kDqRows = 256;   // query rows per workgroup
+constexpr int kDqKeyTile = 32; // keys per LDS tile
 
+// One workgroup = 8 waves = 256 query rows; wave w owns 32 rows: their Q and dO rows sit in
+// registers as MFMA B operands, dQ^T accumulates in registers.  32-key tiles of K and V stream
+// through four LDS buffers with direct-to-LDS loads.  Scores are transposed (S^T = K Q^T,
+// dP^T = V dO^T) exactly as in the forward kernel, so dS^T is the B operand of
+// dQ^T += K^T dS^T whose A operand is the K tile read through the transposing LDS fetch.
+// Inside a wave the matrix unit runs one tile ahead of the vector ALU: the 16 MFMAs of
+// S^T(j+1), dP^T(j+1) carry the exp2 / dS arithmetic of tile j in their shadow, then come the 8
+// MFMAs of dQ^T for tile j.
 template <int D, bool GENERAL>
 __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
-  constexpr int TILE_BYTES = kDqKeyTile * D * 2;
+  constexpr int ROWB = D * 2;
+  constexpr int TILE_BYTES = kDqKeyTile * ROWB;
+  constexpr int NBUF = 4;
 
-  __shared__ __attribute__((aligned(16))) char s_k[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char s_v[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) int s_seg[2][kDqKeyTile];
-  __shared__ __attribute__((aligned(16))) int s_pre[2][kDqKeyTile];
+  __shared__ __attribute__((aligned(16))) char s_k[NBUF][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char s_v[NBUF][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) int s_seg[NBUF][kDqKeyTile];
+  __shared__ __attribute__((aligned(16))) int s_pre[NBUF][kDqKeyTile];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[20];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
   const int nqt = (a.Lq + kDqRows - 1) / kDqRows;
   int hh, qt;
@@ -532,6 +557,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   const int qi_c = min(qi, a.Lq - 1);
   const BiasArgs& bs = a.bias;
   const int flags = bs.flags;
+  const bool wave_on = qw < a.Lq;
 
   bf16x8 qf[KS], dof[KS];
   {
@@ -545,7 +571,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   }
   const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
   const float Lraw = a.lse[row];
-  const float lse2 = (Lraw == RA_NEG_INF) ? __builtin_inff() : Lraw * kLog2e;
+  const float neg_lse2 = (Lraw == RA_NEG_INF) ? RA_NEG_INF : -Lraw * kLog2e;  // fully masked row: P = 0
   const float delta = a.delta[row];
   f32x16 acc[DB];
 #pragma unroll
@@ -563,6 +589,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.kv_seg + b * bs.kv_seg_sb : nullptr;
   const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.kv_pre + b * bs.kv_pre_sb : nullptr;
 
+  // ---- which key tiles does this workgroup visit ------------------------------------------------
   const int ntiles = (a.Lk + kDqKeyTile - 1) / kDqKeyTile;
   const int q_rows_hi = min(q0 + kDqRows, a.Lq) - 1;
   int j_lo, j_hi;
@@ -613,11 +640,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     __syncthreads();
     n_act = s_red[16];
   }
-
-  const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
-  const bf16_t* vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
-  TileStage<D, kDqKeyTile, kDqThreads> kst, vst;
-  int seg_r = 0, pre_r = 0;
+  const int n = n_act;
 
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
@@ -628,95 +651,245 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     segbit = 0;
     return j_lo + i;
   };
-  auto issue_loads = [&](int j) {
-    kst.load(kbase, a.k.sl, j * kDqKeyTile, a.Lk, tid);
-    vst.load(vbase, a.v.sl, j * kDqKeyTile, a.Lk, tid);
+
+  // ---- global -> LDS: every wave moves 4 of a tile's 32 rows of K and of V ---------------------
+  const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
+  const bf16_t* vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
+  constexpr int CPR = D / 8;   // 16-byte chunks per row
+  constexpr int RPW = 4;       // rows per wave per tile
+  // D = 128: one load instruction = 4 rows; D = 64: lanes 0..31 cover the wave's 4 rows
+  const bool ld_lane_on = (lane / CPR) < RPW;
+  const int ld_row = RPW * wave + (lane / CPR) % RPW;
+  const int ld_chunk = ((tile_off<D>(ld_row, lane % CPR) - ld_row * ROWB) >> 4) * 8;
+  const unsigned k_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.k.sl + ld_chunk) * 2);
+  const unsigned v_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.v.sl + ld_chunk) * 2);
+  int seg_r = 0, pre_r = 0;
+  auto issue_tile = [&](int j, int buf) {
+    const int k0 = j * kDqKeyTile;
+    const unsigned k_dst = RA_LDS_ADDR(&s_k[0][0]) + buf * TILE_BYTES + wave_u * RPW * ROWB;
+    const unsigned v_dst = RA_LDS_ADDR(&s_v[0][0]) + buf * TILE_BYTES + wave_u * RPW * ROWB;
+    if (ld_lane_on) {
+      if (k0 + kDqKeyTile <= a.Lk) {
+        global_to_lds16_s(kbase + (long long)(k0 + RPW * wave_u) * a.k.sl, k_voff, k_dst);
+        global_to_lds16_s(vbase + (long long)(k0 + RPW * wave_u) * a.v.sl, v_voff, v_dst);
+      } else {  // last, partial tile: rows past the end repeat the last row (masked later)
+        const int gr = min(k0 + ld_row, a.Lk - 1);
+        global_to_lds16(kbase + (long long)gr * a.k.sl + ld_chunk, k_dst);
+        global_to_lds16(vbase + (long long)gr * a.v.sl + ld_chunk, v_dst);
+      }
+    }
     if (GENERAL && tid < kDqKeyTile) {
-      int kk = min(j * kDqKeyTile + tid, a.Lk - 1);
+      int kk = min(k0 + tid, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
     }
   };
-
-  int sb0 = 0;
-  if (n_act > 0) issue_loads(tile_at(0, sb0));
-
-  for (int i = 0; i < n_act; ++i) {
-    const int buf = i & 1;
-    kst.store(s_k[buf], tid);
-    vst.store(s_v[buf], tid);
+  auto store_ids = [&](int buf) {
     if (GENERAL && tid < kDqKeyTile) {
       s_seg[buf][tid] = seg_r;
       s_pre[buf][tid] = pre_r;
     }
+  };
+
+  // per-lane LDS offsets of the operand fetches
+  int noff[KS];
+#pragma unroll
+  for (int ss = 0; ss < KS; ++ss) noff[ss] = tile_off<D>(l32, 2 * ss + g);
+  int toff[DB][2];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int j = lane & 15;
+      const int trow = 4 * g + (j >> 2) + 8 * h2;
+      const int tcol = 32 * db + 16 * ((lane >> 4) & 1) + 4 * (j & 3);
+      toff[db][h2] = tile_off<D>(trow, tcol >> 3) + ((tcol & 4) << 1);
+    }
+  auto nat_frag = [&](const char* tile, int ss) { return *(const bf16x8*)(tile + noff[ss]); };
+  auto tr_frag = [&](const char* tile, int ks, int db) {
+    const lds_char* p0 = (const lds_char*)(tile + 16 * ks * ROWB + toff[db][0]);
+    const lds_char* p1 = (const lds_char*)(tile + 16 * ks * ROWB + toff[db][1]);
+    bf16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p0);
+    bf16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p1);
+    return __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  auto tile_class = [&](int i, int& kt0, int& segbit) -> int {
+    kt0 = tile_at(i, segbit) * kDqKeyTile;
+    if (flags & RA_BIAS_PREFIX) return 2;
+    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off + kt0,
+                        bs.kv_off + kt0 + kDqKeyTile - 1);
+  };
+  auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
+    bool nb = (cls & 2) || (kt0 + kDqKeyTile > a.Lk);
+    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
+    return nb;
+  };
+  constexpr int PF = 2;
+  auto compute_s_dp = [&](f32x16& S, f32x16& P, const char* kt, const char* vt) {
+    bf16x8 fr[2 * KS];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      S[r] = 0.f;
+      P[r] = 0.f;
+    }
+#pragma unroll
+    for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? vt : kt, op >> 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 2 * KS; ++op) {
+      if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? vt : kt, (op + PF) >> 1);
+      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dof[op >> 1], P, 0, 0, 0);
+      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], S, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto compute_dq = [&](const bf16x8 (&dsf)[2], const char* kt) {
+    bf16x8 fr[2 * DB];
+#pragma unroll
+    for (int op = 0; op < PF; ++op) fr[op] = tr_frag(kt, op / DB, op % DB);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 2 * DB; ++op) {
+      if (op + PF < 2 * DB) fr[op + PF] = tr_frag(kt, (op + PF) / DB, (op + PF) % DB);
+      acc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dsf[op / DB], acc[op % DB], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto prepare = [&](f32x16& S, int kt0, int segbit, int cls, int ids_buf) {
+    TileBias tb;
+    tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
+    if (GENERAL) {
+      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
+      if (segbit) tb.flags |= RA_BIAS_SEGMENT;
+    }
+    tb.window = bs.window;
+    tb.slope2 = slope2;
+    const int var0 = kt0 + 4 * g;
+    tb.var_limit = a.Lk - var0;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] *= a.scale2;
+    const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
+    apply_bias<true>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
+  };
+
+  // ---- prologue: tiles 0, 1, 2 in flight; S^T(0), dP^T(0) computed ------------------------------
+  {
+    int sbu;
+    if (n > 0) {
+      issue_tile(tile_at(0, sbu), 0);
+      store_ids(0);
+    }
+    if (n > 1) {
+      issue_tile(tile_at(1, sbu), 1);
+      store_ids(1);
+    }
+    if (n > 2) issue_tile(tile_at(2, sbu), 2);  // its ids are stored at the top of iteration 0
+  }
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+
+  // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
+  // range: they take the fused path without any per-tile classification.
+  int plain_lo = 0, plain_hi = 0;
+  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT)))) {
+    int lo, hi;
+    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kDqKeyTile,
+                         kDqKeyTile, lo, hi);
+    plain_lo = max(lo - j_lo, 0);
+    plain_hi = min(hi - j_lo, n);
+  }
+
+  f32x16 s_a, p_a, s_b, p_b;
+  bool cur_valid = false, cur_scaled = false;
+  if (n > 0 && wave_on) {
+    int kt0, segbit;
+    const int cls = tile_class(0, kt0, segbit);
+    if (!(cls & 1)) {
+      cur_valid = true;
+      compute_s_dp(s_a, p_a, s_k[0], s_v[0]);
+      cur_scaled = needs_bias(kt0, segbit, cls);
+      if (cur_scaled) prepare(s_a, kt0, segbit, cls, 0);
+    }
+  }
+
+  // one iteration; (SC, PC) hold S^T(i), dP^T(i); (SN, PN) receive tile i+1.  Tile j lives in LDS
+  // buffer j % 4; iteration i reads tiles i (transposed) and i+1, tile i+2 is landing, and the
+  // buffer of tile i-1 is refilled with tile i+3.
+  auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
+    constexpr int PH = decltype(phase)::value;
+    constexpr int PH1 = (PH + 1) % NBUF, PH2 = (PH + 2) % NBUF, PH3 = (PH + 3) % NBUF;
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+2 is in LDS
+    if (i + 2 < n) store_ids(PH2);       // ids of tile i+2 arrived with it
     __syncthreads();
-    int cur_segbit;
-    const int j = tile_at(i, cur_segbit);
-    if (i + 1 < n_act) {
-      int nb;
-      issue_loads(tile_at(i + 1, nb));
+    if (i + 3 < n) {
+      int sbu;
+      issue_tile(tile_at(i + 3, sbu), PH3);
     }
-    if (qw >= a.Lq) continue;
-    const int kt0 = j * kDqKeyTile;
-    const int qlo = bs.q_off + qw, qhi = qlo + 31;
-
+    const char* kc = s_k[PH];
+    const char* kn = s_k[PH1];
+    const char* vn = s_v[PH1];
+    int nkt0 = 0, nsegbit = 0, ncls = 1;
+    bool nxt_valid = false, nxt_scaled = false;
+    if (i + 1 >= plain_lo && i + 1 < plain_hi) {
+      nxt_valid = true;
+    } else if (i + 1 < n && wave_on) {
+      ncls = tile_class(i + 1, nkt0, nsegbit);
+      nxt_valid = !(ncls & 1);
+      nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
+    }
+    bf16x8 dsf[2];
+    if (cur_valid && nxt_valid && !cur_scaled) {
+      // ---- fused: S^T(i+1), dP^T(i+1) MFMAs with the dS arithmetic of tile i in their shadow -----
+      bf16x8 fr[2 * KS];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int kb0 = kt0 + 32 * kb;
-      if (kb0 >= a.Lk) continue;
-      const int klo = bs.kv_off + kb0, khi = klo + 31;
-      const int cls = (flags & RA_BIAS_PREFIX) ? 2 : classify_pos(flags, bs.window, qlo, qhi, klo, khi);
-      if (cls & 1) continue;
-      TileBias tb;
-      tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
-      if (GENERAL) {
-        tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
-        if (cur_segbit) tb.flags |= RA_BIAS_SEGMENT;
-      }
-      tb.window = bs.window;
-      tb.slope2 = slope2;
-      const int var0 = kb0 + 4 * g;
-      tb.var_limit = a.Lk - var0;
-      const bool ragged = kb0 + 32 > a.Lk;
-
-      f32x16 sacc, pacc;
+      for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        sacc[r] = 0.f;
-        pacc[r] = 0.f;
-      }
+      for (int op = 0; op < 2 * KS; ++op) {
+        if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? vn : kn, (op + PF) >> 1);
+        if (op < 2) {
+          f32x16 z;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        bf16x8 ka = frag_nat<D>(s_k[buf], 32 * kb + l32, s, g);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[s], sacc, 0, 0, 0);
-      }
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        bf16x8 va = frag_nat<D>(s_v[buf], 32 * kb + l32, s, g);
-        pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, dof[s], pacc, 0, 0, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[r] *= a.scale2;
-      if (tb.flags != 0 || ragged) {
-        const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
-        apply_bias<true>(sacc, tb, rel0, q_seg, q_pre, &s_seg[buf][32 * kb + 4 * g],
-                         &s_pre[buf][32 * kb + 4 * g]);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = fast_exp2(sacc[r] - lse2);
-        pacc[r] = p * (pacc[r] - delta);
-      }
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const bf16x8 dsf = pack8(pacc, 8 * ks);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          bf16x8 kt = frag_tr<D>(s_k[buf], 32 * kb + 16 * ks, 32 * db, lane);
-          acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kt, dsf, acc[db], 0, 0, 0);
+          for (int r = 0; r < 16; ++r) z[r] = 0.f;
+          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dof[op >> 1], z, 0, 0, 0);
+          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], z, 0, 0, 0);
+        } else {
+          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dof[op >> 1], PN, 0, 0, 0);
+          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN, 0, 0, 0);
         }
+        constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+        if (op * EPO < 16) {
+#pragma unroll
+          for (int e = 0; e < EPO; ++e) {
+            const int r = op * EPO + e;
+            const float p = fast_exp2(fmaf(SC[r], a.scale2, neg_lse2));
+            dsf[r >> 3][r & 7] = (bf16_t)(p * (PC[r] - delta));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      compute_dq(dsf, kc);
+    } else {
+      if (nxt_valid) compute_s_dp(SN, PN, kn, vn);
+      if (cur_valid) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float t = cur_scaled ? SC[r] + neg_lse2 : fmaf(SC[r], a.scale2, neg_lse2);
+          dsf[r >> 3][r & 7] = (bf16_t)(fast_exp2(t) * (PC[r] - delta));
+        }
+        compute_dq(dsf, kc);
       }
     }
+    if (nxt_scaled) prepare(SN, nkt0, nsegbit, ncls, PH1);
+    cur_valid = nxt_valid;
+    cur_scaled = nxt_scaled;
+  };
+
+  for (int i = 0; i < n; i += 4) {
+    iteration(std::integral_constant<int, 0>{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(std::integral_constant<int, 1>{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(std::integral_constant<int, 2>{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(std::integral_constant<int, 3>{}, i + 3, s_b, p_b, s_a, p_a);
   }
 
   if (q_valid) {
@@ -733,6 +906,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
 // ------------------------------------------------------------------------------------------------
 // fp32 accumulator -> bf16 gradient in the caller's layout
 // ------------------------------------------------------------------------------------------------

@@ -283,6 +283,34 @@ RA_DEV void key_tile_range(int flags, int window, int qlo, int qhi, int kv_off, 
   lo = min(max(lo, 0), hi);
 }
 
+// Range [lo, hi) of T-sized key tiles in which EVERY score of queries [qlo, qhi] is unmasked by
+// the positional terms (so no elementwise test is needed), tile j = positions kv_off + T*j + [0, T).
+RA_DEV void key_tile_plain_range(int flags, int window, int qlo, int qhi, int kv_off, int ntiles, int T,
+                                 int& lo, int& hi) {
+  lo = 0;
+  hi = ntiles;
+  if (flags & RA_BIAS_CAUSAL) hi = min(hi, floor_div(qlo - kv_off - (T - 1), T) + 1);
+  if (flags & RA_BIAS_WINDOW) {
+    lo = max(lo, floor_div(qhi - window - kv_off, T) + 1);
+    if (!(flags & RA_BIAS_CAUSAL)) hi = min(hi, ceil_div(qlo + window - kv_off - (T - 1), T));
+  }
+  hi = max(hi, 0);
+  lo = min(max(lo, 0), hi);
+}
+// Mirror image: T-sized query tiles all of whose scores against keys [klo, khi] are unmasked.
+RA_DEV void query_tile_plain_range(int flags, int window, int klo, int khi, int q_off, int ntiles, int T,
+                                   int& lo, int& hi) {
+  lo = 0;
+  hi = ntiles;
+  if (flags & RA_BIAS_CAUSAL) lo = max(lo, ceil_div(khi - q_off, T));
+  if (flags & RA_BIAS_WINDOW) {
+    hi = min(hi, ceil_div(klo + window - q_off - (T - 1), T));
+    if (!(flags & RA_BIAS_CAUSAL)) lo = max(lo, floor_div(khi - window - q_off, T) + 1);
+  }
+  hi = max(hi, 0);
+  lo = min(max(lo, 0), hi);
+}
+
 // Same for the query side: tiles of queries that can see keys at positions [klo, khi].
 RA_DEV void query_tile_range(int flags, int window, int klo, int khi, int q_off, int ntiles, int T,
                              int& lo, int& hi) {

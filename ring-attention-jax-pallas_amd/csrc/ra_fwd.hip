@@ -360,6 +360,17 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     }
   };
 
+  // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
+  // range: they take the fused path without any per-tile classification.
+  int plain_lo = 0, plain_hi = 0;
+  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT)))) {
+    int lo, hi;
+    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kKeyTile,
+                         kKeyTile, lo, hi);
+    plain_lo = max(lo - j_lo, 0);
+    plain_hi = min(hi - j_lo, n);
+  }
+
   // per-tile state handed from one iteration to the next
   f32x16 sa[2], sb[2];
   bool cur_valid = false, cur_scaled = false;
@@ -389,12 +400,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     const char* kt = s_k[PAR ^ 1];
     const char* vt = s_v[PAR];
     int nkt0 = 0, nsegbit = 0, ncls = 1;
-    bool nxt_valid = false;
-    if (i + 1 < n && wave_on) {
+    bool nxt_valid = false, nxt_scaled = false;
+    if (i + 1 >= plain_lo && i + 1 < plain_hi) {
+      nxt_valid = true;
+    } else if (i + 1 < n && wave_on) {
       ncls = tile_class(i + 1, nkt0, nsegbit);
       nxt_valid = !(ncls & 1);
+      nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
     }
-    const bool nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
     float nxt_mx = RA_NEG_INF;
     bf16x8 pfrag[4];
     if (cur_valid) update_reference(cur_mx);
