@@ -25,6 +25,14 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
 
+# HBM bytes per launch (read + written) of the step kernels, measured with
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script (`--copy-probe` gives the
+# 1 GiB copy the counters are scaled by: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Profiler counters
+# cannot be read from inside a timed run, so the figures are carried here.
+MEASURED_HBM_BYTES_PER_LAUNCH = {
+    "C3b": {"fwd_step_kernel": 1.288e9, "dkdv_kernel": 2.402e9, "dq_kernel": 1.433e9},
+}
+
 WORKLOADS = {
     # name: (B, H, D, S, ring, bias, std, description)
     "C3b": dict(B=1, H=32, D=128, S=131072, n=8, bias="causal", std=1.0,
@@ -120,6 +128,8 @@ def main():
     ap.add_argument("--workload", default="C3b", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain elementwise copy of 1 GiB (calibrates HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE GPU: the ring is emulated on a single MI355X and there is no "
@@ -259,7 +269,8 @@ def main():
         ach = kern[dom]["flops"] / kern[dom]["ms"] / 1e9
         result["roofline"] = {"bound": "mfma", "kernel": names[dom], "achieved": round(ach, 2),
                               "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                              "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None}
+                              "frac": round(ach / PEAK_BF16_TFLOPS, 4),
+                              "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(args.workload, {}).get(names[dom])}
         result["kernels"] = kernels
         # rank 7's share (the last query shard against all 8 KV shards)
         if args.workload == "C3b":
@@ -269,6 +280,14 @@ def main():
             P7 = sum(pairs[(n - 1, ks)] for ks in range(n))
             result["rank7_share"] = {"fwd_tflops": round(4.0 * D * P7 * B * H / f_ms / 1e9, 2),
                                      "bwd_tflops": round(10.0 * D * P7 * B * H / b_ms / 1e9, 2)}
+
+    if args.copy_probe:
+        # a kernel of known traffic (reads 1 GiB, writes 1 GiB) for scaling profiler byte counters
+        src = torch.ones(1 << 28, device=dev, dtype=torch.float32)
+        for _ in range(3):
+            dst = src * 1.0
+        torch.cuda.synchronize()
+        del src, dst
 
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(D)

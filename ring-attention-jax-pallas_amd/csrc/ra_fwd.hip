@@ -393,10 +393,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of K_{i+1}, V_i is in LDS
     if (!(RA_ABLATE & 8)) __syncthreads();
     RA_PROF_MARK(i, 2);
-    if (!(RA_ABLATE & 1)) {
-      if (i + 2 < n) issue_k(tile_at(i + 2, sb_unused), PAR);
-      if (i + 1 < n) issue_v(tile_at(i + 1, sb_unused), PAR ^ 1);
-    }
+    auto issue_next = [&]() {
+      if (!(RA_ABLATE & 1)) {
+        if (i + 2 < n) issue_k(tile_at(i + 2, sb_unused), PAR);
+        if (i + 1 < n) issue_v(tile_at(i + 1, sb_unused), PAR ^ 1);
+      }
+    };
     const char* kt = s_k[PAR ^ 1];
     const char* vt = s_v[PAR];
     int nkt0 = 0, nsegbit = 0, ncls = 1;
@@ -410,11 +412,13 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     }
     float nxt_mx = RA_NEG_INF;
     bf16x8 pfrag[4];
+    const bool fused = cur_valid && nxt_valid && !cur_scaled;
+    if (!fused) issue_next();  // the fused path issues the loads inside its second MFMA block
     if (cur_valid) update_reference(cur_mx);
     const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
 
     RA_PROF_MARK(i, 3);
-    if (cur_valid && nxt_valid && !cur_scaled) {
+    if (fused) {
       // ---- fused path: S(i+1) MFMAs with the exp2 / sum / pack of tile i in their shadow -------
       float rs0 = 0.f, rs1 = 0.f;
       {
@@ -466,6 +470,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
           if (op + PF < 4 * DB) fr[op + PF] = pv_op_frag(vt, op + PF);
           if (!(RA_ABLATE & 4)) oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
           else oacc[op % DB][op / DB] += (float)fr[op][0] * (float)pfrag[op / DB][0];
+          if (op == 1) issue_next();  // direct-to-LDS loads of K_{i+2}, V_{i+1}: issue cost hidden behind the MFMAs
 #pragma unroll
           for (int e = 0; e < EPO; e += 2) {
             const int el = op * EPO + e;
