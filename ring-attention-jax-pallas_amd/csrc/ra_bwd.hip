@@ -7,7 +7,7 @@
 //    P and dS are then directly the A operands of dV = P^T dO and dK = dS^T Q, whose B
 //    operands come from the Q / dO tiles through the transposing LDS read.
 //  * dq_kernel: a wave owns 32 queries (Q and dO operands in registers) and streams
-//    64-key tiles of K and V through LDS.  Scores are produced transposed (S^T = K Q^T),
+//    32-key tiles of K and V through four LDS buffers.  Scores are produced transposed (S^T = K Q^T),
 //    exactly as in the forward kernel, so dS^T is the B operand of dQ^T = K^T dS^T.
 // Plus the elementwise delta = rowsum(out * dout) and the fp32 -> bf16 gradient cast.
 #include <type_traits>
