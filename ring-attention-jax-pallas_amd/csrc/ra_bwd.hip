@@ -58,10 +58,11 @@ constexpr int kQTile = 32;  // queries per LDS tile in dkdv_kernel
 // One workgroup = 4 waves = 128 keys; every wave owns 32 keys for the whole kernel: their K
 // and V rows sit in registers as MFMA B operands and the 32 x D dK and dV accumulators in
 // accumulation registers (one wave per SIMD, 512 registers).  32-query tiles of Q and dO are
-// streamed through three LDS buffers with direct-to-LDS loads.  Inside a wave the matrix unit
-// runs one tile ahead of the vector ALU: the 16 MFMAs of S(i+1) = Q K^T and dP(i+1) = dO V^T
-// carry, in their shadow, the exp2 / dS arithmetic of tile i; then come the 16 MFMAs of
-// dV += P(i)^T dO and dK += dS(i)^T Q.
+// streamed through four LDS buffers with direct-to-LDS loads.  Iteration i, after its barrier,
+// first runs the 16 MFMAs of dV += P(i-1)^T dO, dK += dS(i-1)^T Q, whose operands were already
+// visible before the barrier (so their fetch straddles it and the next tile's loads, row
+// statistics and bookkeeping issue in their shadow), then the 16 MFMAs of S(i+1) = Q K^T and
+// dP(i+1) = dO V^T with the exp2 / dS arithmetic of tile i in theirs.
 template <int D, bool GENERAL>
 __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   constexpr int NT = 256;
@@ -71,12 +72,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   constexpr int ROWB = D * 2;
   constexpr int TILE_BYTES = kQTile * ROWB;
 
-  __shared__ __attribute__((aligned(16))) char s_q[3][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char s_do[3][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) float s_lse[3][kQTile];
-  __shared__ __attribute__((aligned(16))) float s_delta[3][kQTile];
-  __shared__ __attribute__((aligned(16))) int s_seg[3][kQTile];
-  __shared__ __attribute__((aligned(16))) int s_pre[3][kQTile];
+  __shared__ __attribute__((aligned(16))) char s_q[4][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char s_do[4][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) float s_lse[4][kQTile];
+  __shared__ __attribute__((aligned(16))) float s_delta[4][kQTile];
+  __shared__ __attribute__((aligned(16))) int s_seg[4][kQTile];
+  __shared__ __attribute__((aligned(16))) int s_pre[4][kQTile];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[12];
@@ -381,7 +382,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     plain_hi = min(hi - i_lo, n);
   }
 
-  f32x16 s_a, p_a, s_b, p_b, s_c, p_c;
+  plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);
+  plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
+
+  f32x16 s_a, p_a, s_b, p_b;
   bool cur_valid = false, cur_scaled = false;
   if (n > 0 && wave_on) {
     int qt0, segbit;
@@ -393,26 +397,40 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       if (cur_scaled) prepare(s_a, qt0, segbit, cls, 0);
     }
   }
+  // P(i-1) and dS(i-1), packed in pairs, waiting for their dV / dK products
+  u32x4 pfw[2], dsw[2];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) pfw[0][e] = pfw[1][e] = dsw[0][e] = dsw[1][e] = 0u;
+  bool pend_valid = false;
+  auto pack2 = [&](float x0, float x1) -> unsigned {
+    bf16x2 t;
+    t[0] = (bf16_t)x0;
+    t[1] = (bf16_t)x1;
+    return __builtin_bit_cast(unsigned, t);
+  };
 
   RA_PROF_DECL
-  // one iteration; (SC, PC) hold S(i), dP(i) on entry, (SN, PN) receive S(i+1), dP(i+1).
-  // Tile j lives in LDS buffer j % 3 = PH for j = i.
+  // Generic iteration; (SC, PC) hold S(i), dP(i) on entry, (SN, PN) receive S(i+1), dP(i+1).
+  // Tile j lives in LDS buffer j % 4 = PH for j = i.
   auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
-    constexpr int PH1 = (PH + 1) % 3, PH2 = (PH + 2) % 3;
-    RA_PROF_MARK(i, 1);
+    constexpr int PHP = (PH + 3) % 4, PH1 = (PH + 1) % 4, PH2 = (PH + 2) % 4;
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+1 is in LDS
     if (i + 1 < n) store_rows(PH1);      // its per-row lse / delta / ids arrived with it
     __syncthreads();
-    RA_PROF_MARK(i, 2);
     if (i + 2 < n) {
       int sbu;
       issue_tile(tile_at(i + 2, sbu), PH2);
     }
-    const char* qc = s_q[PH];
-    const char* doc = s_do[PH];
-    const char* qn = s_q[PH1];
-    const char* don = s_do[PH1];
+    if (pend_valid) {
+      bf16x8 pf[2], dsf[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        pf[ks] = __builtin_bit_cast(bf16x8, pfw[ks]);
+        dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
+      }
+      compute_dkdv(pf, dsf, s_q[PHP], s_do[PHP]);
+    }
     int nqt0 = 0, nsegbit = 0, ncls = 1;
     bool nxt_valid = false, nxt_scaled = false;
     if (i + 1 >= plain_lo && i + 1 < plain_hi) {
@@ -422,77 +440,162 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       nxt_valid = !(ncls & 1);
       nxt_scaled = nxt_valid && needs_bias(nqt0, nsegbit, ncls);
     }
-    bf16x8 pf[2], dsf[2];
-    // per-row statistics of tile i: this lane's 16 query rows are 8*bb + 4*g + c
-    f32x4 L4[4], D4[4];
+    if (nxt_valid) compute_s_dp(SN, PN, s_q[PH1], s_do[PH1]);
     if (cur_valid) {
+      // per-row statistics of tile i: this lane's 16 query rows are 8*bb + 4*g + c
+      f32x4 L4[4], D4[4];
 #pragma unroll
       for (int bb = 0; bb < 4; ++bb) {
         L4[bb] = *(const f32x4*)&s_lse[PH][8 * bb + 4 * g];
         D4[bb] = *(const f32x4*)&s_delta[PH][8 * bb + 4 * g];
       }
-    }
-    RA_PROF_MARK(i, 3);
-    if (cur_valid && nxt_valid && !cur_scaled) {
-      // ---- fused: S(i+1), dP(i+1) MFMAs with P(i), dS(i) arithmetic in their shadow -------------
-      bf16x8 fr[2 * KS];
 #pragma unroll
-      for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? don : qn, op >> 1);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int r = 0; r < 16; r += 2) {
+        float p[2], ds[2];
 #pragma unroll
-      for (int op = 0; op < 2 * KS; ++op) {
-        if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? don : qn, (op + PF) >> 1);
-        if (op < 2) {
-          // first link of each chain starts from a zero accumulator
-          f32x16 z;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) z[r] = 0.f;
-          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], z, 0, 0, 0);
-          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], z, 0, 0, 0);
-        } else {
-          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], PN, 0, 0, 0);
-          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], SN, 0, 0, 0);
+        for (int e = 0; e < 2; ++e) {
+          const float lse2 = L4[(r + e) >> 2][(r + e) & 3];
+          const float t = cur_scaled ? SC[r + e] - lse2 : fmaf(SC[r + e], a.scale2, -lse2);
+          p[e] = fast_exp2(t);
+          ds[e] = p[e] * (PC[r + e] - D4[(r + e) >> 2][(r + e) & 3]);
         }
-        constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
-        if (op * EPO < 16) {
-#pragma unroll
-          for (int e = 0; e < EPO; ++e) {
-            const int r = op * EPO + e;
-            const float p = fast_exp2(fmaf(SC[r], a.scale2, -L4[r >> 2][r & 3]));
-            const float ds = p * (PC[r] - D4[r >> 2][r & 3]);
-            pf[r >> 3][r & 7] = (bf16_t)p;
-            dsf[r >> 3][r & 7] = (bf16_t)ds;
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      RA_PROF_MARK(i, 4);
-      compute_dkdv(pf, dsf, qc, doc);
-      RA_PROF_MARK(i, 5);
-    } else {
-      if (nxt_valid) compute_s_dp(SN, PN, qn, don);
-      if (cur_valid) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float t = cur_scaled ? SC[r] - L4[r >> 2][r & 3] : fmaf(SC[r], a.scale2, -L4[r >> 2][r & 3]);
-          const float p = fast_exp2(t);
-          const float ds = p * (PC[r] - D4[r >> 2][r & 3]);
-          pf[r >> 3][r & 7] = (bf16_t)p;
-          dsf[r >> 3][r & 7] = (bf16_t)ds;
-        }
-        compute_dkdv(pf, dsf, qc, doc);
+        pfw[r >> 3][(r & 7) >> 1] = pack2(p[0], p[1]);
+        dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
       }
     }
+    pend_valid = cur_valid;
     if (nxt_scaled) prepare(SN, nqt0, nsegbit, ncls, PH1);
     cur_valid = nxt_valid;
     cur_scaled = nxt_scaled;
-    RA_PROF_MARK(i, 6);
   };
 
-  for (int i = 0; i < n; i += 3) {
-    iteration(std::integral_constant<int, 0>{}, i, s_a, p_a, s_b, p_b);
-    if (i + 1 < n) iteration(std::integral_constant<int, 1>{}, i + 1, s_b, p_b, s_c, p_c);
-    if (i + 2 < n) iteration(std::integral_constant<int, 2>{}, i + 2, s_c, p_c, s_a, p_a);
+  // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+2
+  // exists, so there is nothing to classify and no flag to consult.
+  auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
+    constexpr int PH = decltype(phase)::value;
+    constexpr int PHP = (PH + 3) % 4, PH1 = (PH + 1) % 4, PH2 = (PH + 2) % 4;
+    const char* qp = s_q[PHP];
+    const char* dop = s_do[PHP];
+    const char* qn = s_q[PH1];
+    const char* don = s_do[PH1];
+    RA_PROF_MARK(i, 1);
+    // operands of the dV / dK products come from tile i-1, visible since two barriers ago
+    bf16x8 frb[4 * DB];
+#pragma unroll
+    for (int op = 0; op < PF; ++op) frb[op] = tr_frag((op & 1) ? qp : dop, op / (2 * DB), (op >> 1) % DB);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+1 is in LDS
+    store_rows(PH1);
+    __syncthreads();
+    RA_PROF_MARK(i, 2);
+    bf16x8 pf[2], dsf[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      pf[ks] = __builtin_bit_cast(bf16x8, pfw[ks]);
+      dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
+    }
+    f32x4 L4[4], D4[4];
+    bf16x8 fra[2 * KS];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 4 * DB; ++op) {
+      if (op + PF < 4 * DB) {
+        const int o2 = op + PF;
+        frb[o2] = tr_frag((o2 & 1) ? qp : dop, o2 / (2 * DB), (o2 >> 1) % DB);
+      } else {
+        // the first operands of the S / dP products ride behind the last dV / dK MFMAs
+        const int o2 = op + PF - 4 * DB;
+        fra[o2] = nat_frag((o2 & 1) ? don : qn, o2 >> 1);
+      }
+      const int ks = op / (2 * DB), db = (op >> 1) % DB;
+      if (op & 1) dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[ks], frb[op], dk[db], 0, 0, 0);
+      else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], frb[op], dv[db], 0, 0, 0);
+      if (op == 0) {  // next tile's loads: their issue hides behind the MFMAs
+        int sbu;
+        issue_tile(tile_at(i + 2, sbu), PH2);
+      }
+      if (op >= 2 && op < 6) {  // row statistics of tile i for the arithmetic below
+        const int bb = op - 2;
+        L4[bb] = *(const f32x4*)&s_lse[PH][8 * bb + 4 * g];
+        D4[bb] = *(const f32x4*)&s_delta[PH][8 * bb + 4 * g];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    RA_PROF_MARK(i, 3);
+    // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA
+    float p_prev = 0.f, ds_prev = 0.f;
+#pragma unroll
+    for (int op = 0; op < 2 * KS; ++op) {
+      if (op + PF < 2 * KS) fra[op + PF] = nat_frag(((op + PF) & 1) ? don : qn, (op + PF) >> 1);
+      if (op < 2) {
+        // first link of each chain starts from a zero accumulator
+        f32x16 z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], z, 0, 0, 0);
+        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], z, 0, 0, 0);
+      } else {
+        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], PN, 0, 0, 0);
+        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], SN, 0, 0, 0);
+      }
+      constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+      if (op * EPO < 16) {
+#pragma unroll
+        for (int e = 0; e < EPO; ++e) {
+          const int r = op * EPO + e;
+          float p = fast_exp2(fmaf(SC[r], a.scale2, -L4[r >> 2][r & 3]));
+          float ds = p * (PC[r] - D4[r >> 2][r & 3]);
+          asm volatile("" : "+v"(p), "+v"(ds));  // pins the arithmetic between two MFMAs
+          if (r & 1) {
+            unsigned pw = pack2(p_prev, p), dw = pack2(ds_prev, ds);
+            asm volatile("" : "+v"(pw), "+v"(dw));
+            pfw[r >> 3][(r & 7) >> 1] = pw;
+            dsw[r >> 3][(r & 7) >> 1] = dw;
+          }
+          p_prev = p;
+          ds_prev = ds;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    RA_PROF_MARK(i, 4);
+  };
+
+  // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
+  // plain stretch in whole groups of four, generic iterations for the rest.  Every wave runs n
+  // iterations in total, so the barrier counts agree.
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using P2 = std::integral_constant<int, 2>;
+  using P3 = std::integral_constant<int, 3>;
+  const int plain_end = min(plain_hi - 1, n - 2);  // iteration i is plain for plain_lo < i < plain_end
+  int i = 0;
+  for (; i < n && !(i > plain_lo && i + 4 <= plain_end); i += 4) {
+    iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+  }
+  for (; i + 4 <= plain_end; i += 4) {
+    plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+  }
+  for (; i < n; i += 4) {
+    iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+  }
+  if (pend_valid) {  // products of the last tile
+    bf16x8 pf[2], dsf[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      pf[ks] = __builtin_bit_cast(bf16x8, pfw[ks]);
+      dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
+    }
+    const int last = (n - 1) & 3;
+    compute_dkdv(pf, dsf, s_q[last], s_do[last]);
   }
 
   RA_PROF_DUMP;
