@@ -18,6 +18,16 @@
 #define RA_ABLATE_B 0  // timing experiments only: bit mask of loop parts to leave out
 #endif
 
+#if defined(RA_PROFILE) && defined(PROF_DQ)
+#define RA_PROFQ_DECL RA_PROF_DECL
+#define RA_PROFQ_MARK(i, id) RA_PROF_MARK(i, id)
+#define RA_PROFQ_DUMP RA_PROF_DUMP
+#else
+#define RA_PROFQ_DECL
+#define RA_PROFQ_MARK(i, id) do { } while (0)
+#define RA_PROFQ_DUMP do { } while (0)
+#endif
+
 namespace ra {
 
 constexpr int kBwdMaxListTiles = 2048;
@@ -74,8 +84,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 
   __shared__ __attribute__((aligned(16))) char s_q[4][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char s_do[4][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) float s_lse[4][kQTile];
-  __shared__ __attribute__((aligned(16))) float s_delta[4][kQTile];
+  // per-row statistics as one more 16-wide slice of the contraction: row r of s_aug[buf][0]
+  // holds -lse / sm_scale split into three bf16 terms (then zeros), s_aug[buf][1] holds -delta
+  // likewise; multiplied with a (1, 1, 1, 0, ...) column they put S - lse / sm_scale and
+  // dP - delta straight into the accumulators
+  __shared__ __attribute__((aligned(16))) bf16_t s_aug[4][2][kQTile][16];
   __shared__ __attribute__((aligned(16))) int s_seg[4][kQTile];
   __shared__ __attribute__((aligned(16))) int s_pre[4][kQTile];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
@@ -255,11 +268,27 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       if (GENERAL && q_pre) pre_r = q_pre[qq];
     }
   };
+  auto split3 = [&](float x) -> bf16x4 {  // x = t[0] + t[1] + t[2] exactly (3 x 8 mantissa bits)
+    bf16x4 t;
+    t[0] = (bf16_t)x;
+    const float r1 = x - (float)t[0];
+    t[1] = (bf16_t)r1;
+    t[2] = (bf16_t)(r1 - (float)t[1]);
+    t[3] = (bf16_t)0.f;
+    return t;
+  };
+  const float inv_sm_scale = 1.0f / a.sm_scale;
   auto store_rows = [&](int buf) {
     if (tid < kQTile) {
-      // log2 domain; a fully masked row (lse = -inf) becomes +inf so that its P is 0
-      s_lse[buf][tid] = (lse_r == RA_NEG_INF) ? __builtin_inff() : lse_r * kLog2e;
-      s_delta[buf][tid] = delta_r;
+      // a fully masked row (lse = -inf) gets -inf so that its P is 0
+      bf16x4 tl = split3(-lse_r * inv_sm_scale);
+      if (lse_r == RA_NEG_INF) {
+        tl[0] = (bf16_t)RA_NEG_INF;
+        tl[1] = (bf16_t)0.f;
+        tl[2] = (bf16_t)0.f;
+      }
+      *(bf16x4*)&s_aug[buf][0][tid][0] = tl;
+      *(bf16x4*)&s_aug[buf][1][tid][0] = split3(-delta_r);
       if (GENERAL) {
         s_seg[buf][tid] = seg_r;
         s_pre[buf][tid] = pre_r;
@@ -303,14 +332,20 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
     return nb;
   };
+  bf16x8 ones3;  // B operand of the statistics slice: (1, 1, 1, 0, ...) in the first half-wave
+#pragma unroll
+  for (int e = 0; e < 8; ++e) ones3[e] = (bf16_t)((g == 0 && e < 3) ? 1.f : 0.f);
+  auto aug_frag = [&](int buf, int which) { return *(const bf16x8*)&s_aug[buf][which][l32][8 * g]; };
   // S = Q K^T and dP = dO V^T of one tile, nothing interleaved
   constexpr int PF = 3;
-  auto compute_s_dp = [&](f32x16& S, f32x16& P, const char* qt, const char* dot) {
+  auto compute_s_dp = [&](f32x16& S, f32x16& P, const char* qt, const char* dot, int buf) {
     bf16x8 fr[2 * KS];
+    {
+      f32x16 z;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      S[r] = 0.f;
-      P[r] = 0.f;
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aug_frag(buf, 0), ones3, z, 0, 0, 0);
+      P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aug_frag(buf, 1), ones3, z, 0, 0, 0);
     }
 #pragma unroll
     for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? dot : qt, op >> 1);
@@ -358,6 +393,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     apply_bias<false>(S, tb, rel0, k_seg, k_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
   };
 
+  // the twelve trailing zeros of every statistics row are written once
+  for (int e = tid; e < 4 * 2 * kQTile * 16 / 2; e += NT) ((unsigned*)&s_aug[0][0][0][0])[e] = 0u;
+  __syncthreads();
+
   // ---- prologue: tiles 0 and 1 in flight, S(0) and dP(0) computed -----------------------------
   if (n > 0) {
     int sbu;
@@ -392,7 +431,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     const int cls = tile_class(0, qt0, segbit);
     if (!(cls & 1)) {
       cur_valid = true;
-      compute_s_dp(s_a, p_a, s_q[0], s_do[0]);
+      compute_s_dp(s_a, p_a, s_q[0], s_do[0], 0);
       cur_scaled = needs_bias(qt0, segbit, cls);
       if (cur_scaled) prepare(s_a, qt0, segbit, cls, 0);
     }
@@ -440,24 +479,16 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       nxt_valid = !(ncls & 1);
       nxt_scaled = nxt_valid && needs_bias(nqt0, nsegbit, ncls);
     }
-    if (nxt_valid) compute_s_dp(SN, PN, s_q[PH1], s_do[PH1]);
+    if (nxt_valid) compute_s_dp(SN, PN, s_q[PH1], s_do[PH1], PH1);
     if (cur_valid) {
-      // per-row statistics of tile i: this lane's 16 query rows are 8*bb + 4*g + c
-      f32x4 L4[4], D4[4];
-#pragma unroll
-      for (int bb = 0; bb < 4; ++bb) {
-        L4[bb] = *(const f32x4*)&s_lse[PH][8 * bb + 4 * g];
-        D4[bb] = *(const f32x4*)&s_delta[PH][8 * bb + 4 * g];
-      }
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float p[2], ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          const float lse2 = L4[(r + e) >> 2][(r + e) & 3];
-          const float t = cur_scaled ? SC[r + e] - lse2 : fmaf(SC[r + e], a.scale2, -lse2);
-          p[e] = fast_exp2(t);
-          ds[e] = p[e] * (PC[r + e] - D4[(r + e) >> 2][(r + e) & 3]);
+          // the accumulators already hold S - lse / sm_scale and dP - delta
+          p[e] = fast_exp2(cur_scaled ? SC[r + e] : SC[r + e] * a.scale2);
+          ds[e] = p[e] * PC[r + e];
         }
         pfw[r >> 3][(r & 7) >> 1] = pack2(p[0], p[1]);
         dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
@@ -469,8 +500,42 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     cur_scaled = nxt_scaled;
   };
 
+  // Loads of the plain stretch: consecutive full tiles, so the wave-uniform global addresses
+  // advance by a constant and stay in scalar registers.
+  const bf16_t* q_run = qbase;
+  const bf16_t* do_run = dobase;
+  const float* lse_run = lse_row;
+  const float* delta_run = delta_row;
+  const unsigned q_dst0 = RA_LDS_ADDR(&s_q[0][0]) + wave_u * 8 * ROWB;
+  const unsigned do_dst0 = RA_LDS_ADDR(&s_do[0][0]) + wave_u * 8 * ROWB;
+  auto seek_plain = [&](int tile) {
+    q_run = qbase + (long long)(tile * kQTile + 8 * wave_u) * a.q.sl;
+    do_run = dobase + (long long)(tile * kQTile + 8 * wave_u) * a.dout.sl;
+    lse_run = lse_row + tile * kQTile;
+    delta_run = delta_row + tile * kQTile;
+  };
+  auto issue_plain = [&](int buf) {
+    if (NLD == 2) {
+      global_to_lds16_s_x2(q_run, q_voff[0], q_run + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1],
+                           q_dst0 + buf * TILE_BYTES);
+      global_to_lds16_s_x2(do_run, do_voff[0], do_run + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1],
+                           do_dst0 + buf * TILE_BYTES);
+    } else {
+      global_to_lds16_s(q_run, q_voff[0], q_dst0 + buf * TILE_BYTES);
+      global_to_lds16_s(do_run, do_voff[0], do_dst0 + buf * TILE_BYTES);
+    }
+    if (tid < kQTile) {  // consumed in store_rows, one iteration later
+      lse_r = lse_run[tid];
+      delta_r = delta_run[tid];
+    }
+    q_run += (long long)kQTile * a.q.sl;
+    do_run += (long long)kQTile * a.dout.sl;
+    lse_run += kQTile;
+    delta_run += kQTile;
+  };
+
   // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+2
-  // exists, so there is nothing to classify and no flag to consult.
+  // exists and is complete, so there is nothing to classify and no flag to consult.
   auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
     constexpr int PHP = (PH + 3) % 4, PH1 = (PH + 1) % 4, PH2 = (PH + 2) % 4;
@@ -493,8 +558,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       pf[ks] = __builtin_bit_cast(bf16x8, pfw[ks]);
       dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
     }
-    f32x4 L4[4], D4[4];
     bf16x8 fra[2 * KS];
+    bf16x8 fa_s, fa_p;  // statistics slices of tile i+1
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int op = 0; op < 4 * DB; ++op) {
@@ -509,41 +574,37 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       const int ks = op / (2 * DB), db = (op >> 1) % DB;
       if (op & 1) dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[ks], frb[op], dk[db], 0, 0, 0);
       else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], frb[op], dv[db], 0, 0, 0);
-      if (op == 0) {  // next tile's loads: their issue hides behind the MFMAs
-        int sbu;
-        issue_tile(tile_at(i + 2, sbu), PH2);
-      }
-      if (op >= 2 && op < 6) {  // row statistics of tile i for the arithmetic below
-        const int bb = op - 2;
-        L4[bb] = *(const f32x4*)&s_lse[PH][8 * bb + 4 * g];
-        D4[bb] = *(const f32x4*)&s_delta[PH][8 * bb + 4 * g];
+      if (op == 0) issue_plain(PH2);  // next tile's loads: their issue hides behind the MFMAs
+      if (op == 4 * DB - PF - 1) {
+        fa_s = aug_frag(PH1, 0);
+        fa_p = aug_frag(PH1, 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     RA_PROF_MARK(i, 3);
-    // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA
+    // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA.  The
+    // chains start with the statistics slice.
     float p_prev = 0.f, ds_prev = 0.f;
+    {
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_s, ones3, z, 0, 0, 0);
+      PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_p, ones3, z, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PF < 2 * KS) fra[op + PF] = nat_frag(((op + PF) & 1) ? don : qn, (op + PF) >> 1);
-      if (op < 2) {
-        // first link of each chain starts from a zero accumulator
-        f32x16 z;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], z, 0, 0, 0);
-        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], z, 0, 0, 0);
-      } else {
-        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], PN, 0, 0, 0);
-        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], SN, 0, 0, 0);
-      }
+      if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], PN, 0, 0, 0);
+      else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], SN, 0, 0, 0);
       constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
       if (op * EPO < 16) {
 #pragma unroll
         for (int e = 0; e < EPO; ++e) {
           const int r = op * EPO + e;
-          float p = fast_exp2(fmaf(SC[r], a.scale2, -L4[r >> 2][r & 3]));
-          float ds = p * (PC[r] - D4[r >> 2][r & 3]);
+          float p = fast_exp2(SC[r] * a.scale2);
+          float ds = p * PC[r];
           asm volatile("" : "+v"(p), "+v"(ds));  // pins the arithmetic between two MFMAs
           if (r & 1) {
             unsigned pw = pack2(p_prev, p), dw = pack2(ds_prev, ds);
@@ -567,7 +628,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   using P1 = std::integral_constant<int, 1>;
   using P2 = std::integral_constant<int, 2>;
   using P3 = std::integral_constant<int, 3>;
-  const int plain_end = min(plain_hi - 1, n - 2);  // iteration i is plain for plain_lo < i < plain_end
+  // iteration i is plain for plain_lo < i < plain_end (tile i+2 must exist and be complete)
+  const int plain_end = min(min(plain_hi - 1, n - 2), a.Lq / kQTile - i_lo - 2);
   int i = 0;
   for (; i < n && !(i > plain_lo && i + 4 <= plain_end); i += 4) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
@@ -575,6 +637,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
     if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
   }
+  if (i + 4 <= plain_end) seek_plain(i_lo + i + 2);
   for (; i + 4 <= plain_end; i += 4) {
     plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
     plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
@@ -623,19 +686,19 @@ constexpr int kDqKeyTile = 32; // keys per LDS tile
 
 // One workgroup = 8 waves = 256 query rows; wave w owns 32 rows: their Q and dO rows sit in
 // registers as MFMA B operands, dQ^T accumulates in registers.  32-key tiles of K and V stream
-// through four LDS buffers with direct-to-LDS loads.  Scores are transposed (S^T = K Q^T,
-// dP^T = V dO^T) exactly as in the forward kernel, so dS^T is the B operand of
-// dQ^T += K^T dS^T whose A operand is the K tile read through the transposing LDS fetch.
-// Inside a wave the matrix unit runs one tile ahead of the vector ALU: the 16 MFMAs of
-// S^T(j+1), dP^T(j+1) carry the exp2 / dS arithmetic of tile j in their shadow, then come the 8
-// MFMAs of dQ^T for tile j.
+// through six LDS buffers with direct-to-LDS loads issued three tiles ahead.  Scores are
+// transposed (S^T = K Q^T, dP^T = V dO^T) exactly as in the forward kernel, so dS^T is the B
+// operand of dQ^T += K^T dS^T whose A operand is the K tile read through the transposing LDS
+// fetch.  Iteration i, after its barrier, first runs the 8 MFMAs of dQ^T for tile i-1 (operands
+// visible before the barrier, so their fetch straddles it), then the 16 MFMAs of S^T(i+1),
+// dP^T(i+1) with the exp2 / dS arithmetic of tile i in their shadow.
 template <int D, bool GENERAL>
 __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
   constexpr int ROWB = D * 2;
   constexpr int TILE_BYTES = kDqKeyTile * ROWB;
-  constexpr int NBUF = 4;
+  constexpr int NBUF = 6;
 
   __shared__ __attribute__((aligned(16))) char s_k[NBUF][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char s_v[NBUF][TILE_BYTES];
@@ -902,6 +965,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     plain_hi = min(hi - j_lo, n);
   }
 
+  plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);
+  plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
+
   f32x16 s_a, p_a, s_b, p_b;
   bool cur_valid = false, cur_scaled = false;
   if (n > 0 && wave_on) {
@@ -914,13 +980,25 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       if (cur_scaled) prepare(s_a, kt0, segbit, cls, 0);
     }
   }
+  // dS^T(i-1), packed in pairs, waiting for its dQ^T product
+  u32x4 dsw[2];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) dsw[0][e] = dsw[1][e] = 0u;
+  bool pend_valid = false;
+  auto pack2 = [&](float x0, float x1) -> unsigned {
+    bf16x2 t;
+    t[0] = (bf16_t)x0;
+    t[1] = (bf16_t)x1;
+    return __builtin_bit_cast(unsigned, t);
+  };
 
-  // one iteration; (SC, PC) hold S^T(i), dP^T(i); (SN, PN) receive tile i+1.  Tile j lives in LDS
-  // buffer j % 4; iteration i reads tiles i (transposed) and i+1, tile i+2 is landing, and the
-  // buffer of tile i-1 is refilled with tile i+3.
+  RA_PROFQ_DECL
+  // Generic iteration; (SC, PC) hold S^T(i), dP^T(i); (SN, PN) receive tile i+1.  Tile j lives in
+  // LDS buffer j % 6; iteration i reads tiles i-1 (transposed) and i+1, tile i stays for the next
+  // iteration, tile i+2 is landing, tile i+3 is issued.
   auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
-    constexpr int PH1 = (PH + 1) % NBUF, PH2 = (PH + 2) % NBUF, PH3 = (PH + 3) % NBUF;
+    constexpr int PHP = (PH + NBUF - 1) % NBUF, PH1 = (PH + 1) % NBUF, PH2 = (PH + 2) % NBUF, PH3 = (PH + 3) % NBUF;
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+2 is in LDS
     if (i + 2 < n) store_ids(PH2);       // ids of tile i+2 arrived with it
     __syncthreads();
@@ -928,9 +1006,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       int sbu;
       issue_tile(tile_at(i + 3, sbu), PH3);
     }
-    const char* kc = s_k[PH];
-    const char* kn = s_k[PH1];
-    const char* vn = s_v[PH1];
+    if (pend_valid) {
+      bf16x8 dsf[2];
+      dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
+      dsf[1] = __builtin_bit_cast(bf16x8, dsw[1]);
+      compute_dq(dsf, s_k[PHP]);
+    }
     int nkt0 = 0, nsegbit = 0, ncls = 1;
     bool nxt_valid = false, nxt_scaled = false;
     if (i + 1 >= plain_lo && i + 1 < plain_hi) {
@@ -940,61 +1021,156 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       nxt_valid = !(ncls & 1);
       nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
     }
-    bf16x8 dsf[2];
-    if (cur_valid && nxt_valid && !cur_scaled) {
-      // ---- fused: S^T(i+1), dP^T(i+1) MFMAs with the dS arithmetic of tile i in their shadow -----
-      bf16x8 fr[2 * KS];
+    if (nxt_valid) compute_s_dp(SN, PN, s_k[PH1], s_v[PH1]);
+    if (cur_valid) {
 #pragma unroll
-      for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int r = 0; r < 16; r += 2) {
+        float ds[2];
 #pragma unroll
-      for (int op = 0; op < 2 * KS; ++op) {
-        if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? vn : kn, (op + PF) >> 1);
-        if (op < 2) {
-          f32x16 z;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) z[r] = 0.f;
-          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dof[op >> 1], z, 0, 0, 0);
-          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], z, 0, 0, 0);
-        } else {
-          if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dof[op >> 1], PN, 0, 0, 0);
-          else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN, 0, 0, 0);
+        for (int e = 0; e < 2; ++e) {
+          const float t = cur_scaled ? SC[r + e] + neg_lse2 : fmaf(SC[r + e], a.scale2, neg_lse2);
+          ds[e] = fast_exp2(t) * (PC[r + e] - delta);
         }
-        constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
-        if (op * EPO < 16) {
-#pragma unroll
-          for (int e = 0; e < EPO; ++e) {
-            const int r = op * EPO + e;
-            const float p = fast_exp2(fmaf(SC[r], a.scale2, neg_lse2));
-            dsf[r >> 3][r & 7] = (bf16_t)(p * (PC[r] - delta));
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      compute_dq(dsf, kc);
-    } else {
-      if (nxt_valid) compute_s_dp(SN, PN, kn, vn);
-      if (cur_valid) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float t = cur_scaled ? SC[r] + neg_lse2 : fmaf(SC[r], a.scale2, neg_lse2);
-          dsf[r >> 3][r & 7] = (bf16_t)(fast_exp2(t) * (PC[r] - delta));
-        }
-        compute_dq(dsf, kc);
+        dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
       }
     }
+    pend_valid = cur_valid;
     if (nxt_scaled) prepare(SN, nkt0, nsegbit, ncls, PH1);
     cur_valid = nxt_valid;
     cur_scaled = nxt_scaled;
   };
 
-  for (int i = 0; i < n; i += 4) {
-    iteration(std::integral_constant<int, 0>{}, i, s_a, p_a, s_b, p_b);
-    if (i + 1 < n) iteration(std::integral_constant<int, 1>{}, i + 1, s_b, p_b, s_a, p_a);
-    if (i + 2 < n) iteration(std::integral_constant<int, 2>{}, i + 2, s_a, p_a, s_b, p_b);
-    if (i + 3 < n) iteration(std::integral_constant<int, 3>{}, i + 3, s_b, p_b, s_a, p_a);
+  // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
+  // exists, so there is nothing to classify and no flag to consult.  Waves 4..7 take the
+  // iteration's barrier between the two MFMA blocks instead of before them (see below).
+  const bool late_half = wave_u >= 4;
+  auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
+    constexpr int PH = decltype(phase)::value;
+    constexpr int PHP = (PH + NBUF - 1) % NBUF, PH1 = (PH + 1) % NBUF, PH3 = (PH + 3) % NBUF;
+    const char* kp = s_k[PHP];
+    const char* kn = s_k[PH1];
+    const char* vn = s_v[PH1];
+    // operands of the dQ^T product come from tile i-1, visible since two barriers ago
+    RA_PROFQ_MARK(i, 1);
+    bf16x8 frb[2 * DB];
+#pragma unroll
+    for (int op = 0; op < PF; ++op) frb[op] = tr_frag(kp, op / DB, op % DB);
+    if (!late_half) {
+      // all loads but the two of tile i+2 have landed: this wave's share of tile i+1 is in LDS
+      if (GENERAL) __builtin_amdgcn_s_waitcnt(0x0f70);
+      else __builtin_amdgcn_s_waitcnt(0x0f72);
+      __syncthreads();
+    }
+    RA_PROFQ_MARK(i, 2);
+    bf16x8 dsf[2];
+    dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
+    dsf[1] = __builtin_bit_cast(bf16x8, dsw[1]);
+    bf16x8 fra[2 * KS];
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int op = 0; op < 2 * DB; ++op) {
+      if (op + PF < 2 * DB) {
+        frb[op + PF] = tr_frag(kp, (op + PF) / DB, (op + PF) % DB);
+      } else if (!late_half) {
+        // the first operands of the S^T / dP^T products ride behind the last dQ^T MFMAs
+        const int o2 = op + PF - 2 * DB;
+        fra[o2] = nat_frag((o2 & 1) ? vn : kn, o2 >> 1);
+      }
+      acc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frb[op], dsf[op / DB], acc[op % DB], 0, 0, 0);
+      if (op == 0) {  // next loads: their issue hides behind the MFMAs
+        int sbu;
+        issue_tile(tile_at(i + 3, sbu), PH3);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (late_half) {
+      // this half of the workgroup meets the barrier here, so that on every SIMD one wave runs
+      // its dQ^T block while the other runs its S^T / dP^T block.  Tiles i+2 and i+3 may still
+      // be in flight (two loads each).
+      if (GENERAL) __builtin_amdgcn_s_waitcnt(0x0f70);
+      else __builtin_amdgcn_s_waitcnt(0x0f74);
+      __syncthreads();
+#pragma unroll
+      for (int op = 0; op < PF; ++op) fra[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
+    }
+    RA_PROFQ_MARK(i, 3);
+    float ds_prev = 0.f;
+#pragma unroll
+    for (int op = 0; op < 2 * KS; ++op) {
+      if (op + PF < 2 * KS) fra[op + PF] = nat_frag(((op + PF) & 1) ? vn : kn, (op + PF) >> 1);
+      if (op < 2) {
+        f32x16 z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], dof[op >> 1], z, 0, 0, 0);
+        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], qf[op >> 1], z, 0, 0, 0);
+      } else {
+        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], dof[op >> 1], PN, 0, 0, 0);
+        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], qf[op >> 1], SN, 0, 0, 0);
+      }
+      constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+      if (op * EPO < 16) {
+#pragma unroll
+        for (int e = 0; e < EPO; ++e) {
+          const int r = op * EPO + e;
+          float ds = fast_exp2(fmaf(SC[r], a.scale2, neg_lse2)) * (PC[r] - delta);
+          asm volatile("" : "+v"(ds));  // pins the arithmetic between two MFMAs
+          if (r & 1) {
+            unsigned dw = pack2(ds_prev, ds);
+            asm volatile("" : "+v"(dw));
+            dsw[r >> 3][(r & 7) >> 1] = dw;
+          }
+          ds_prev = ds;
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    RA_PROFQ_MARK(i, 4);
+  };
+
+  // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
+  // plain stretch in whole groups of six, generic iterations for the rest.  Every wave runs n
+  // iterations in total, so the barrier counts agree.
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using P2 = std::integral_constant<int, 2>;
+  using P3 = std::integral_constant<int, 3>;
+  using P4 = std::integral_constant<int, 4>;
+  using P5 = std::integral_constant<int, 5>;
+  const int plain_end = min(plain_hi - 1, n - 3);  // iteration i is plain for plain_lo < i < plain_end
+  int i = 0;
+  for (; i < n && !(i > plain_lo && i + 6 <= plain_end); i += 6) {
+    iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+    if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+    if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+  }
+  for (; i + 6 <= plain_end; i += 6) {
+    plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+    plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+    plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+  }
+  for (; i < n; i += 6) {
+    iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+    if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+    if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+  }
+  if (pend_valid) {  // product of the last tile
+    bf16x8 dsf[2];
+    dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
+    dsf[1] = __builtin_bit_cast(bf16x8, dsw[1]);
+    compute_dq(dsf, s_k[0] + ((n - 1) % NBUF) * TILE_BYTES);
   }
 
+  RA_PROFQ_DUMP;
   if (q_valid) {
     float* dq = a.dq + row * D + 4 * g;
 #pragma unroll
