@@ -549,8 +549,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int op = 0; op < PF; ++op) frb[op] = tr_frag((op & 1) ? qp : dop, op / (2 * DB), (op >> 1) % DB);
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+1 is in LDS
-    store_rows(PH1);
-    __syncthreads();
+    if (!(RA_ABLATE_B & 32)) store_rows(PH1);
+    if (!(RA_ABLATE_B & 4)) __syncthreads();
     RA_PROF_MARK(i, 2);
     bf16x8 pf[2], dsf[2];
 #pragma unroll
@@ -574,7 +574,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       const int ks = op / (2 * DB), db = (op >> 1) % DB;
       if (op & 1) dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[ks], frb[op], dk[db], 0, 0, 0);
       else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], frb[op], dv[db], 0, 0, 0);
-      if (op == 0) issue_plain(PH2);  // next tile's loads: their issue hides behind the MFMAs
+      if (op == 0 && !(RA_ABLATE_B & 16)) issue_plain(PH2);  // next tile's loads: their issue hides behind the MFMAs
       if (op == 4 * DB - PF - 1) {
         fa_s = aug_frag(PH1, 0);
         fa_p = aug_frag(PH1, 1);
@@ -599,7 +599,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], PN, 0, 0, 0);
       else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], SN, 0, 0, 0);
       constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
-      if (op * EPO < 16) {
+      if (op * EPO < 16 && !(RA_ABLATE_B & 8)) {
 #pragma unroll
         for (int e = 0; e < EPO; ++e) {
           const int r = op * EPO + e;
