@@ -65,14 +65,19 @@ __global__ void bwd_delta_kernel(const OutT* out, long long sb, long long sh, lo
 // ------------------------------------------------------------------------------------------------
 constexpr int kQTile = 32;  // queries per LDS tile in dkdv_kernel
 
+// s_waitcnt with only the vector-memory counter set (expcnt, lgkmcnt left at their maxima)
+#define RA_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+
 // One workgroup = 4 waves = 128 keys; every wave owns 32 keys for the whole kernel: their K
-// and V rows sit in registers as MFMA B operands and the 32 x D dK and dV accumulators in
-// accumulation registers (one wave per SIMD, 512 registers).  32-query tiles of Q and dO are
-// streamed through four LDS buffers with direct-to-LDS loads.  Iteration i, after its barrier,
-// first runs the 16 MFMAs of dV += P(i-1)^T dO, dK += dS(i-1)^T Q, whose operands were already
-// visible before the barrier (so their fetch straddles it and the next tile's loads, row
-// statistics and bookkeeping issue in their shadow), then the 16 MFMAs of S(i+1) = Q K^T and
-// dP(i+1) = dO V^T with the exp2 / dS arithmetic of tile i in theirs.
+// and V rows sit in registers as MFMA B operands (K already multiplied by sm_scale * log2(e))
+// and the 32 x D dK and dV accumulators in accumulation registers (one wave per SIMD, 512
+// registers).  32-query tiles of Q and dO stream through six LDS buffers with direct-to-LDS loads
+// requested three tiles ahead; a tile's per-row statistics (-lse * log2(e), -delta) travel next
+// to it and enter the score and dP accumulators as the MFMA chains' initial C operand.
+// Iteration i, after its barrier, first runs the 16 MFMAs of dV += P(i-1)^T dO, dK += dS(i-1)^T Q
+// (operands visible before the barrier, so their fetch straddles it; the next tile's loads and
+// the hand-over of S(i), dP(i) to the vector ALU issue in their shadow), then the 16 MFMAs of
+// S(i+1) = Q K^T and dP(i+1) = dO V^T with the exp2 / dS arithmetic of tile i in theirs.
 template <int D, bool GENERAL>
 __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   constexpr int NT = 256;
@@ -81,16 +86,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   constexpr int KEYS_WG = 128;
   constexpr int ROWB = D * 2;
   constexpr int TILE_BYTES = kQTile * ROWB;
+  constexpr int NB = 6;                    // LDS tile buffers; tile j lives in buffer j % NB
+  constexpr int NSTAT = GENERAL ? 4 : 2;   // per-row words that travel with a tile
+  constexpr int STAT_BYTES = 4 * kQTile * 4;
 
-  __shared__ __attribute__((aligned(16))) char s_q[4][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char s_do[4][TILE_BYTES];
-  // per-row statistics as one more 16-wide slice of the contraction: row r of s_aug[buf][0]
-  // holds -lse / sm_scale split into three bf16 terms (then zeros), s_aug[buf][1] holds -delta
-  // likewise; multiplied with a (1, 1, 1, 0, ...) column they put S - lse / sm_scale and
-  // dP - delta straight into the accumulators
-  __shared__ __attribute__((aligned(16))) bf16_t s_aug[4][2][kQTile][16];
-  __shared__ __attribute__((aligned(16))) int s_seg[4][kQTile];
-  __shared__ __attribute__((aligned(16))) int s_pre[4][kQTile];
+  __shared__ __attribute__((aligned(16))) char s_q[NB][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char s_do[NB][TILE_BYTES];
+  // per tile and row: -lse * log2(e) (-inf for a fully masked row), -delta, segment id, prefix flag
+  __shared__ __attribute__((aligned(16))) char s_stat[NB][STAT_BYTES];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[12];
@@ -111,6 +114,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   const bool wave_on = kw < a.Lk;
 
   // ---- resident key-side operands ----------------------------------------------------------
+  // K is scaled once, here, so that the score MFMAs deliver S * sm_scale * log2(e) directly;
+  // its rounding to bf16 perturbs a probability by a few 1e-3 relative, like the rounding of P.
   bf16x8 kf[KS], vf[KS];
   int k_seg = 0, k_pre = 0;
   {
@@ -119,7 +124,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     const bf16_t* vp = a.v.ptr + b * a.v.sb + h * a.v.sh + (long long)ki * a.v.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      kf[s] = *(const bf16x8*)(kp + 16 * s);
+      const bf16x8 kr = *(const bf16x8*)(kp + 16 * s);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) kf[s][e] = (bf16_t)((float)kr[e] * a.scale2);
       vf[s] = *(const bf16x8*)(vp + 16 * s);
     }
     if (GENERAL && (flags & RA_BIAS_SEGMENT)) k_seg = bs.kv_seg[b * bs.kv_seg_sb + ki];
@@ -218,11 +225,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   // physical chunk l % CPR of row l / CPR and fetches the logical chunk the XOR layout puts there
   const bf16_t* qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
   const bf16_t* dobase = a.dout.ptr + b * a.dout.sb + h * a.dout.sh;
-  const float* lse_row = a.lse + ((long long)b * a.H + h) * a.Lq;
-  const float* delta_row = a.delta + ((long long)b * a.H + h) * a.Lq;
   constexpr int CPR = D / 8;
   constexpr int RPI = 64 / CPR;
   constexpr int NLD = 8 / RPI;
+  constexpr int LPT = 2 * NLD + 1;  // vector-memory instructions per wave and tile
   int ld_row[NLD], ld_off[NLD];
   unsigned q_voff[NLD], do_voff[NLD];  // per-lane byte offsets inside a group of RPI rows
 #pragma unroll
@@ -234,14 +240,34 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     q_voff[t] = (unsigned)(((long long)(lane / CPR) * a.q.sl + ld_off[t]) * 2);
     do_voff[t] = (unsigned)(((long long)(lane / CPR) * a.dout.sl + ld_off[t]) * 2);
   }
-  float lse_r = 0.f, delta_r = 0.f;
-  int seg_r = 0, pre_r = 0;
-  auto issue_tile = [&](int it, int buf) {
+  // The per-row words of a tile: lane l of every wave fetches word class (l / 8) % NSTAT of row
+  // 8 * wave + l % 8 into a register (lanes 32..63 repeat lanes 0..31), and writes it, converted,
+  // to s_stat when the tile is awaited.  The load is issued as inline assembly like the tile
+  // loads, so the compiler adds no waits of its own; three registers rotate (tiles i+1 .. i+3).
+  const int st_class = (lane >> 3) & (NSTAT - 1);
+  const int st_row = 8 * wave + (lane & 7);
+  const char* st_src;
+  {
+    const long long rowbase = ((long long)b * a.H + h) * a.Lq;
+    const char* c0 = (const char*)(a.lse + rowbase);
+    const char* c1 = (const char*)(a.delta + rowbase);
+    const char* c2 = GENERAL && q_seg ? (const char*)q_seg : c0;
+    const char* c3 = GENERAL && q_pre ? (const char*)q_pre : c0;
+    st_src = st_class == 0 ? c0 : (st_class == 1 ? c1 : (st_class == 2 ? c2 : c3));
+  }
+  const unsigned st_dst = (unsigned)(st_class * (kQTile * 4) + st_row * 4);
+  const float st_mul = st_class == 0 ? -kLog2e : -1.0f;
+  const float st_fix = st_class == 0 ? RA_NEG_INF : 0.f;
+  unsigned xr[3] = {0u, 0u, 0u};
+  auto load_stat = [&](const char* p, unsigned& x) {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(x) : "v"(p) : "memory");
+  };
+  auto issue_tile = [&](int it, int buf, unsigned& x) {
     const int q0 = it * kQTile;
     const unsigned q_dst = RA_LDS_ADDR(&s_q[0][0]) + buf * TILE_BYTES + wave_u * 8 * ROWB;
     const unsigned do_dst = RA_LDS_ADDR(&s_do[0][0]) + buf * TILE_BYTES + wave_u * 8 * ROWB;
-    if (RA_ABLATE_B & 1) {
-    } else if (q0 + kQTile <= a.Lq) {
+    load_stat(st_src + 4ll * min(q0 + st_row, a.Lq - 1), x);
+    if (q0 + kQTile <= a.Lq) {
       // wave-uniform row addresses in scalar registers, per-lane part in one VGPR
       const bf16_t* qs = qbase + (long long)(q0 + 8 * wave_u) * a.q.sl;
       const bf16_t* ds = dobase + (long long)(q0 + 8 * wave_u) * a.dout.sl;
@@ -260,40 +286,17 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
         global_to_lds16(dobase + (long long)gr * a.dout.sl + ld_off[t], do_dst + RPI * t * ROWB);
       }
     }
-    if (tid < kQTile && !(RA_ABLATE_B & 2)) {  // values are consumed in store_rows, one iteration later
-      const int qq = min(q0 + tid, a.Lq - 1);
-      lse_r = lse_row[qq];
-      delta_r = delta_row[qq];
-      if (GENERAL && q_seg) seg_r = q_seg[qq];
-      if (GENERAL && q_pre) pre_r = q_pre[qq];
-    }
   };
-  auto split3 = [&](float x) -> bf16x4 {  // x = t[0] + t[1] + t[2] exactly (3 x 8 mantissa bits)
-    bf16x4 t;
-    t[0] = (bf16_t)x;
-    const float r1 = x - (float)t[0];
-    t[1] = (bf16_t)r1;
-    t[2] = (bf16_t)(r1 - (float)t[1]);
-    t[3] = (bf16_t)0.f;
-    return t;
-  };
-  const float inv_sm_scale = 1.0f / a.sm_scale;
-  auto store_rows = [&](int buf) {
-    if (tid < kQTile) {
-      // a fully masked row (lse = -inf) gets -inf so that its P is 0
-      bf16x4 tl = split3(-lse_r * inv_sm_scale);
-      if (lse_r == RA_NEG_INF) {
-        tl[0] = (bf16_t)RA_NEG_INF;
-        tl[1] = (bf16_t)0.f;
-        tl[2] = (bf16_t)0.f;
-      }
-      *(bf16x4*)&s_aug[buf][0][tid][0] = tl;
-      *(bf16x4*)&s_aug[buf][1][tid][0] = split3(-delta_r);
-      if (GENERAL) {
-        s_seg[buf][tid] = seg_r;
-        s_pre[buf][tid] = pre_r;
-      }
-    }
+  // converts the awaited tile's per-row word and publishes it (the caller has waited for it)
+  auto store_stat = [&](int buf, unsigned& x) {
+    asm volatile("" : "+v"(x));
+    // lse -> -lse * log2(e), but -inf for a fully masked row (lse = -inf) so that its P is 0;
+    // delta -> -delta, but 0 for the NaN that a fully masked output row produces
+    float v = __uint_as_float(x) * st_mul;
+    v = (v < __builtin_inff()) ? v : st_fix;
+    unsigned o = __float_as_uint(v);
+    if (GENERAL) o = st_class >= 2 ? x : o;
+    *(unsigned*)(&s_stat[0][0] + buf * STAT_BYTES + st_dst) = o;
   };
 
   // per-lane LDS offsets of the operand fetches (the tile buffer and the 16-row step fold into
@@ -319,6 +322,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     bf16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p1);
     return __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+  // the statistics of the 16 queries an accumulator lane holds: rows 8 * bb + 4 * g + {0..3}
+  const char* stat_rd = &s_stat[0][0] + 16 * g;
+  auto stat_chunk = [&](int buf, int which, int bb) {
+    return *(const f32x4*)(stat_rd + buf * STAT_BYTES + which * (kQTile * 4) + 32 * bb);
+  };
 
   // positional class of this wave's 32 keys against query tile index i
   auto tile_class = [&](int i, int& qt0, int& segbit) -> int {
@@ -332,29 +340,29 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
     return nb;
   };
-  bf16x8 ones3;  // B operand of the statistics slice: (1, 1, 1, 0, ...) in the first half-wave
-#pragma unroll
-  for (int e = 0; e < 8; ++e) ones3[e] = (bf16_t)((g == 0 && e < 3) ? 1.f : 0.f);
-  auto aug_frag = [&](int buf, int which) { return *(const bf16x8*)&s_aug[buf][which][l32][8 * g]; };
-  // S = Q K^T and dP = dO V^T of one tile, nothing interleaved
-  constexpr int PF = 3;
+  constexpr int PFN = 4;  // operand fetches kept in flight ahead of the MFMA that uses them
+  constexpr int PFT = 4;
+  // S * scale2 - lse2 = Q K'^T and dP - delta = dO V^T of one tile, nothing interleaved
   auto compute_s_dp = [&](f32x16& S, f32x16& P, const char* qt, const char* dot, int buf) {
     bf16x8 fr[2 * KS];
-    {
-      f32x16 z;
+    f32x16 cS, cP;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) z[r] = 0.f;
-      S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aug_frag(buf, 0), ones3, z, 0, 0, 0);
-      P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(aug_frag(buf, 1), ones3, z, 0, 0, 0);
+    for (int bb = 0; bb < 4; ++bb) {
+      const f32x4 t0 = stat_chunk(buf, 0, bb), t1 = stat_chunk(buf, 1, bb);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        cS[4 * bb + c] = t0[c];
+        cP[4 * bb + c] = t1[c];
+      }
     }
 #pragma unroll
-    for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? dot : qt, op >> 1);
+    for (int op = 0; op < PFN; ++op) fr[op] = nat_frag((op & 1) ? dot : qt, op >> 1);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
-      if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? dot : qt, (op + PF) >> 1);
-      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], P, 0, 0, 0);
-      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], S, 0, 0, 0);
+      if (op + PFN < 2 * KS) fr[op + PFN] = nat_frag(((op + PFN) & 1) ? dot : qt, (op + PFN) >> 1);
+      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], op == 1 ? cP : P, 0, 0, 0);
+      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], op == 0 ? cS : S, 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -362,12 +370,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   auto compute_dkdv = [&](const bf16x8 (&pf)[2], const bf16x8 (&dsf)[2], const char* qt, const char* dot) {
     bf16x8 fr[4 * DB];
 #pragma unroll
-    for (int op = 0; op < PF; ++op) fr[op] = tr_frag((op & 1) ? qt : dot, op / (2 * DB), (op >> 1) % DB);
+    for (int op = 0; op < PFT; ++op) fr[op] = tr_frag((op & 1) ? qt : dot, op / (2 * DB), (op >> 1) % DB);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int op = 0; op < 4 * DB; ++op) {
-      if (op + PF < 4 * DB) {
-        const int o2 = op + PF;
+      if (op + PFT < 4 * DB) {
+        const int o2 = op + PFT;
         fr[o2] = tr_frag((o2 & 1) ? qt : dot, o2 / (2 * DB), (o2 >> 1) % DB);
       }
       const int ks = op / (2 * DB), db = (op >> 1) % DB;
@@ -376,7 +384,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // scale + bias of a fresh S in place (rows of the accumulator are queries)
+  // bias of a fresh S in place (rows of the accumulator are queries; S is in log2 units already)
   auto prepare = [&](f32x16& S, int qt0, int segbit, int cls, int ids_buf) {
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
@@ -387,27 +395,21 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     tb.window = bs.window;
     tb.slope2 = slope2;
     tb.var_limit = a.Lq - (qt0 + 4 * g);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) S[r] *= a.scale2;
     const int rel0 = (bs.q_off + qt0 + 4 * g) - (bs.kv_off + kw + l32);
-    apply_bias<false>(S, tb, rel0, k_seg, k_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
+    const int* ids = (const int*)(stat_rd + ids_buf * STAT_BYTES);
+    apply_bias<false>(S, tb, rel0, k_seg, k_pre, ids + 2 * kQTile, ids + 3 * kQTile);
   };
 
-  // the twelve trailing zeros of every statistics row are written once
-  for (int e = tid; e < 4 * 2 * kQTile * 16 / 2; e += NT) ((unsigned*)&s_aug[0][0][0][0])[e] = 0u;
-  __syncthreads();
-
-  // ---- prologue: tiles 0 and 1 in flight, S(0) and dP(0) computed -----------------------------
-  if (n > 0) {
+  // ---- prologue: tiles 0, 1, 2 requested, S(0) and dP(0) computed ------------------------------
+  {
     int sbu;
-    issue_tile(tile_at(0, sbu), 0);
-    store_rows(0);
+    if (n > 0) issue_tile(tile_at(0, sbu), 0, xr[0]);
+    if (n > 1) issue_tile(tile_at(1, sbu), 1, xr[1]);
+    if (n > 2) issue_tile(tile_at(2, sbu), 2, xr[2]);  // its statistics are stored in iteration 1
+    __builtin_amdgcn_s_waitcnt(0);
+    if (n > 0) store_stat(0, xr[0]);
+    if (n > 1) store_stat(1, xr[1]);
   }
-  if (n > 1) {
-    int sbu;
-    issue_tile(tile_at(1, sbu), 1);  // its rows are stored at the top of iteration 0
-  }
-  __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
 
   // Ordinals [plain_lo, plain_hi) of the query tiles this wave's keys see completely, unmasked
@@ -420,20 +422,18 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     plain_lo = max(lo - i_lo, 0);
     plain_hi = min(hi - i_lo, n);
   }
-
   plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);
   plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
 
-  f32x16 s_a, p_a, s_b, p_b;
-  bool cur_valid = false, cur_scaled = false;
+  f32x16 s_c, p_c;  // S(i) * scale2 - lse2 and dP(i) - delta of the current tile
+  bool cur_valid = false;
   if (n > 0 && wave_on) {
     int qt0, segbit;
     const int cls = tile_class(0, qt0, segbit);
     if (!(cls & 1)) {
       cur_valid = true;
-      compute_s_dp(s_a, p_a, s_q[0], s_do[0], 0);
-      cur_scaled = needs_bias(qt0, segbit, cls);
-      if (cur_scaled) prepare(s_a, qt0, segbit, cls, 0);
+      compute_s_dp(s_c, p_c, s_q[0], s_do[0], 0);
+      if (needs_bias(qt0, segbit, cls)) prepare(s_c, qt0, segbit, cls, 0);
     }
   }
   // P(i-1) and dS(i-1), packed in pairs, waiting for their dV / dK products
@@ -449,17 +449,23 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   };
 
   RA_PROF_DECL
-  // Generic iteration; (SC, PC) hold S(i), dP(i) on entry, (SN, PN) receive S(i+1), dP(i+1).
-  // Tile j lives in LDS buffer j % 4 = PH for j = i.
-  auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
+  // Generic iteration.  Tile j lives in LDS buffer j % NB = PH for j = i.
+  auto iteration = [&](auto phase, int i) {
     constexpr int PH = decltype(phase)::value;
-    constexpr int PHP = (PH + 3) % 4, PH1 = (PH + 1) % 4, PH2 = (PH + 2) % 4;
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+1 is in LDS
-    if (i + 1 < n) store_rows(PH1);      // its per-row lse / delta / ids arrived with it
-    __syncthreads();
+    constexpr int PHP = (PH + NB - 1) % NB, PH1 = (PH + 1) % NB, PH2 = (PH + 2) % NB, PH3 = (PH + 3) % NB;
+    // this wave's share of tile i+1 is in LDS once at most the loads of tile i+2 are in flight;
+    // the per-row word of tile i+2 (the first load of its group) is published one iteration
+    // before the tile is read
     if (i + 2 < n) {
+      RA_WAIT_VMCNT(LPT - 1);
+      store_stat(PH2, xr[PH2 % 3]);
+    } else {
+      RA_WAIT_VMCNT(0);
+    }
+    __syncthreads();
+    if (i + 3 < n) {
       int sbu;
-      issue_tile(tile_at(i + 2, sbu), PH2);
+      issue_tile(tile_at(i + 3, sbu), PH3, xr[PH3 % 3]);
     }
     if (pend_valid) {
       bf16x8 pf[2], dsf[2];
@@ -470,75 +476,55 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       }
       compute_dkdv(pf, dsf, s_q[PHP], s_do[PHP]);
     }
-    int nqt0 = 0, nsegbit = 0, ncls = 1;
-    bool nxt_valid = false, nxt_scaled = false;
-    if (i + 1 >= plain_lo && i + 1 < plain_hi) {
-      nxt_valid = true;
-    } else if (i + 1 < n && wave_on) {
-      ncls = tile_class(i + 1, nqt0, nsegbit);
-      nxt_valid = !(ncls & 1);
-      nxt_scaled = nxt_valid && needs_bias(nqt0, nsegbit, ncls);
-    }
-    if (nxt_valid) compute_s_dp(SN, PN, s_q[PH1], s_do[PH1], PH1);
     if (cur_valid) {
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float p[2], ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          // the accumulators already hold S - lse / sm_scale and dP - delta
-          p[e] = fast_exp2(cur_scaled ? SC[r + e] : SC[r + e] * a.scale2);
-          ds[e] = p[e] * PC[r + e];
+          p[e] = fast_exp2(s_c[r + e]);
+          ds[e] = p[e] * p_c[r + e];
         }
         pfw[r >> 3][(r & 7) >> 1] = pack2(p[0], p[1]);
         dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
       }
     }
     pend_valid = cur_valid;
-    if (nxt_scaled) prepare(SN, nqt0, nsegbit, ncls, PH1);
+    int nqt0 = 0, nsegbit = 0, ncls = 1;
+    bool nxt_valid = false;
+    if (i + 1 >= plain_lo && i + 1 < plain_hi) {
+      nxt_valid = true;
+      ncls = 0;
+    } else if (i + 1 < n && wave_on) {
+      ncls = tile_class(i + 1, nqt0, nsegbit);
+      nxt_valid = !(ncls & 1);
+    }
+    if (nxt_valid) {
+      compute_s_dp(s_c, p_c, s_q[PH1], s_do[PH1], PH1);
+      if (!(i + 1 >= plain_lo && i + 1 < plain_hi) && needs_bias(nqt0, nsegbit, ncls))
+        prepare(s_c, nqt0, nsegbit, ncls, PH1);
+    }
     cur_valid = nxt_valid;
-    cur_scaled = nxt_scaled;
   };
 
   // Loads of the plain stretch: consecutive full tiles, so the wave-uniform global addresses
   // advance by a constant and stay in scalar registers.
   const bf16_t* q_run = qbase;
   const bf16_t* do_run = dobase;
-  const float* lse_run = lse_row;
-  const float* delta_run = delta_row;
+  const char* st_run = st_src;
   const unsigned q_dst0 = RA_LDS_ADDR(&s_q[0][0]) + wave_u * 8 * ROWB;
   const unsigned do_dst0 = RA_LDS_ADDR(&s_do[0][0]) + wave_u * 8 * ROWB;
   auto seek_plain = [&](int tile) {
     q_run = qbase + (long long)(tile * kQTile + 8 * wave_u) * a.q.sl;
     do_run = dobase + (long long)(tile * kQTile + 8 * wave_u) * a.dout.sl;
-    lse_run = lse_row + tile * kQTile;
-    delta_run = delta_row + tile * kQTile;
-  };
-  auto issue_plain = [&](int buf) {
-    if (NLD == 2) {
-      global_to_lds16_s_x2(q_run, q_voff[0], q_run + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1],
-                           q_dst0 + buf * TILE_BYTES);
-      global_to_lds16_s_x2(do_run, do_voff[0], do_run + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1],
-                           do_dst0 + buf * TILE_BYTES);
-    } else {
-      global_to_lds16_s(q_run, q_voff[0], q_dst0 + buf * TILE_BYTES);
-      global_to_lds16_s(do_run, do_voff[0], do_dst0 + buf * TILE_BYTES);
-    }
-    if (tid < kQTile) {  // consumed in store_rows, one iteration later
-      lse_r = lse_run[tid];
-      delta_r = delta_run[tid];
-    }
-    q_run += (long long)kQTile * a.q.sl;
-    do_run += (long long)kQTile * a.dout.sl;
-    lse_run += kQTile;
-    delta_run += kQTile;
+    st_run = st_src + 4ll * (tile * kQTile + st_row);
   };
 
-  // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+2
+  // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
   // exists and is complete, so there is nothing to classify and no flag to consult.
-  auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
+  auto plain_iteration = [&](auto phase, int i) {
     constexpr int PH = decltype(phase)::value;
-    constexpr int PHP = (PH + 3) % 4, PH1 = (PH + 1) % 4, PH2 = (PH + 2) % 4;
+    constexpr int PHP = (PH + NB - 1) % NB, PH1 = (PH + 1) % NB, PH2 = (PH + 2) % NB, PH3 = (PH + 3) % NB;
     const char* qp = s_q[PHP];
     const char* dop = s_do[PHP];
     const char* qn = s_q[PH1];
@@ -547,10 +533,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     // operands of the dV / dK products come from tile i-1, visible since two barriers ago
     bf16x8 frb[4 * DB];
 #pragma unroll
-    for (int op = 0; op < PF; ++op) frb[op] = tr_frag((op & 1) ? qp : dop, op / (2 * DB), (op >> 1) % DB);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile i+1 is in LDS
-    if (!(RA_ABLATE_B & 32)) store_rows(PH1);
-    if (!(RA_ABLATE_B & 4)) __syncthreads();
+    for (int op = 0; op < PFT; ++op) frb[op] = tr_frag((op & 1) ? qp : dop, op / (2 * DB), (op >> 1) % DB);
+    // all but the loads of tile i+2 have landed: this wave's share of tile i+1 is in LDS.  The
+    // barrier is issued without a fence: the only LDS operations in flight are the PFT operand
+    // fetches above, and what other waves need (the statistics stored half an iteration ago) is
+    // older than those.
+    RA_WAIT_VMCNT(LPT);
+    if (!(RA_ABLATE_B & 4)) asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" : : "n"(2 * PFT) : "memory");
     RA_PROF_MARK(i, 2);
     bf16x8 pf[2], dsf[2];
 #pragma unroll
@@ -559,96 +548,143 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
     }
     bf16x8 fra[2 * KS];
-    bf16x8 fa_s, fa_p;  // statistics slices of tile i+1
+    float sc[16], pc[16];  // S(i), dP(i) handed to the vector ALU
+    f32x16 cS, cP;         // initial accumulator values of S(i+1), dP(i+1)
+    constexpr int NOPS = 4 * DB;
+    constexpr int RPO = 32 / NOPS > 4 ? 32 / NOPS : 4;  // accumulator registers handed over per MFMA
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int op = 0; op < 4 * DB; ++op) {
-      if (op + PF < 4 * DB) {
-        const int o2 = op + PF;
+    for (int op = 0; op < NOPS; ++op) {
+      if (op + PFT < NOPS) {
+        const int o2 = op + PFT;
         frb[o2] = tr_frag((o2 & 1) ? qp : dop, o2 / (2 * DB), (o2 >> 1) % DB);
       } else {
         // the first operands of the S / dP products ride behind the last dV / dK MFMAs
-        const int o2 = op + PF - 4 * DB;
-        fra[o2] = nat_frag((o2 & 1) ? don : qn, o2 >> 1);
+        const int o2 = op + PFT - NOPS;
+        if (o2 < PFN) fra[o2] = nat_frag((o2 & 1) ? don : qn, o2 >> 1);
       }
       const int ks = op / (2 * DB), db = (op >> 1) % DB;
       if (op & 1) dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[ks], frb[op], dk[db], 0, 0, 0);
       else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], frb[op], dv[db], 0, 0, 0);
-      if (op == 0 && !(RA_ABLATE_B & 16)) issue_plain(PH2);  // next tile's loads: their issue hides behind the MFMAs
-      if (op == 4 * DB - PF - 1) {
-        fa_s = aug_frag(PH1, 0);
-        fa_p = aug_frag(PH1, 1);
+      // next tile's loads, one instruction group per MFMA: their issue hides behind the MFMAs
+      if (!(RA_ABLATE_B & 16)) {
+        if (op == 0) {
+          load_stat(st_run, xr[PH3 % 3]);
+          st_run += kQTile * 4;
+        }
+        if (op == 1) {
+          if (NLD == 2) global_to_lds16_s_x2(q_run, q_voff[0], q_run + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1], q_dst0 + PH3 * TILE_BYTES);
+          else global_to_lds16_s(q_run, q_voff[0], q_dst0 + PH3 * TILE_BYTES);
+          q_run += (long long)kQTile * a.q.sl;
+        }
+        if (op == 2) {
+          if (NLD == 2) global_to_lds16_s_x2(do_run, do_voff[0], do_run + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1], do_dst0 + PH3 * TILE_BYTES);
+          else global_to_lds16_s(do_run, do_voff[0], do_dst0 + PH3 * TILE_BYTES);
+          do_run += (long long)kQTile * a.dout.sl;
+        }
+      }
+      // S(i), dP(i) leave the accumulation registers in the first half of the block ...
+#pragma unroll
+      for (int e = 0; e < RPO; ++e) {
+        const int x = op * RPO + e;
+        if (x < 16) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sc[x]) : "a"(s_c[x]));
+        else if (x < 32) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(pc[x - 16]) : "a"(p_c[x - 16]));
+      }
+      // ... and the statistics of tile i+1 enter them in the second half
+      {
+        const int j = op - (NOPS - 8);
+        if (j >= 0) {
+          const f32x4 t = stat_chunk(PH1, j >> 2, j & 3);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            if (j >> 2) cP[4 * (j & 3) + c] = t[c];
+            else cS[4 * (j & 3) + c] = t[c];
+          }
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
     RA_PROF_MARK(i, 3);
-    // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA.  The
-    // chains start with the statistics slice.
-    float p_prev = 0.f, ds_prev = 0.f;
-    {
-      f32x16 z;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) z[r] = 0.f;
-      SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_s, ones3, z, 0, 0, 0);
-      PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_p, ones3, z, 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA, the chain of
+    // an element (exp2, product, packing) spread over consecutive slots
+    float pe[16], de[16];
+    constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
-      if (op + PF < 2 * KS) fra[op + PF] = nat_frag(((op + PF) & 1) ? don : qn, (op + PF) >> 1);
-      if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], PN, 0, 0, 0);
-      else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], SN, 0, 0, 0);
-      constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
-      if (op * EPO < 16 && !(RA_ABLATE_B & 8)) {
+      if (op + PFN < 2 * KS) fra[op + PFN] = nat_frag(((op + PFN) & 1) ? don : qn, (op + PFN) >> 1);
+      if (op & 1) p_c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], op == 1 ? cP : p_c, 0, 0, 0);
+      else s_c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], op == 0 ? cS : s_c, 0, 0, 0);
+      if (op == 2 && !(RA_ABLATE_B & 32)) {
+        // the per-row word of tile i+2 is the oldest load but those of its tile and of tile i+3
+        RA_WAIT_VMCNT(2 * LPT - 1);
+        store_stat(PH2, xr[PH2 % 3]);
+      }
+      if (!(RA_ABLATE_B & 8)) {
 #pragma unroll
         for (int e = 0; e < EPO; ++e) {
           const int r = op * EPO + e;
-          float p = fast_exp2(SC[r] * a.scale2);
-          float ds = p * PC[r];
-          asm volatile("" : "+v"(p), "+v"(ds));  // pins the arithmetic between two MFMAs
-          if (r & 1) {
-            unsigned pw = pack2(p_prev, p), dw = pack2(ds_prev, ds);
-            asm volatile("" : "+v"(pw), "+v"(dw));
-            pfw[r >> 3][(r & 7) >> 1] = pw;
-            dsw[r >> 3][(r & 7) >> 1] = dw;
+          if (r < 16) {
+            pe[r] = fast_exp2(sc[r]);
+            asm volatile("" : "+v"(pe[r]));
           }
-          p_prev = p;
-          ds_prev = ds;
+          if (r >= 1 && r <= 16) {
+            de[r - 1] = pe[r - 1] * pc[r - 1];
+            asm volatile("" : "+v"(de[r - 1]));
+          }
+          if (r >= 2 && r <= 16 && !(r & 1)) {
+            unsigned pw = pack2(pe[r - 2], pe[r - 1]), dw = pack2(de[r - 2], de[r - 1]);
+            asm volatile("" : "+v"(pw), "+v"(dw));
+            pfw[(r - 2) >> 3][((r - 2) & 7) >> 1] = pw;
+            dsw[(r - 2) >> 3][((r - 2) & 7) >> 1] = dw;
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (!(RA_ABLATE_B & 8)) {
+      de[15] = pe[15] * pc[15];
+      pfw[1][3] = pack2(pe[14], pe[15]);
+      dsw[1][3] = pack2(de[14], de[15]);
     }
     RA_PROF_MARK(i, 4);
   };
 
   // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
-  // plain stretch in whole groups of four, generic iterations for the rest.  Every wave runs n
+  // plain stretch in whole groups of six, generic iterations for the rest.  Every wave runs n
   // iterations in total, so the barrier counts agree.
   using P0 = std::integral_constant<int, 0>;
   using P1 = std::integral_constant<int, 1>;
   using P2 = std::integral_constant<int, 2>;
   using P3 = std::integral_constant<int, 3>;
-  // iteration i is plain for plain_lo < i < plain_end (tile i+2 must exist and be complete)
-  const int plain_end = min(min(plain_hi - 1, n - 2), a.Lq / kQTile - i_lo - 2);
+  using P4 = std::integral_constant<int, 4>;
+  using P5 = std::integral_constant<int, 5>;
+  // iteration i is plain for plain_lo < i < plain_end (tile i+3 must exist and be complete)
+  const int plain_end = min(min(plain_hi - 1, n - 3), a.Lq / kQTile - i_lo - 3);
   int i = 0;
-  for (; i < n && !(i > plain_lo && i + 4 <= plain_end); i += 4) {
-    iteration(P0{}, i, s_a, p_a, s_b, p_b);
-    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
-    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
-    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+  for (; i < n && !(i > plain_lo && i + NB <= plain_end); i += NB) {
+    iteration(P0{}, i);
+    if (i + 1 < n) iteration(P1{}, i + 1);
+    if (i + 2 < n) iteration(P2{}, i + 2);
+    if (i + 3 < n) iteration(P3{}, i + 3);
+    if (i + 4 < n) iteration(P4{}, i + 4);
+    if (i + 5 < n) iteration(P5{}, i + 5);
   }
-  if (i + 4 <= plain_end) seek_plain(i_lo + i + 2);
-  for (; i + 4 <= plain_end; i += 4) {
-    plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
-    plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
-    plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
-    plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+  if (i + NB <= plain_end) seek_plain(i_lo + i + 3);
+  for (; i + NB <= plain_end; i += NB) {
+    plain_iteration(P0{}, i);
+    plain_iteration(P1{}, i + 1);
+    plain_iteration(P2{}, i + 2);
+    plain_iteration(P3{}, i + 3);
+    plain_iteration(P4{}, i + 4);
+    plain_iteration(P5{}, i + 5);
   }
-  for (; i < n; i += 4) {
-    iteration(P0{}, i, s_a, p_a, s_b, p_b);
-    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
-    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
-    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+  for (; i < n; i += NB) {
+    iteration(P0{}, i);
+    if (i + 1 < n) iteration(P1{}, i + 1);
+    if (i + 2 < n) iteration(P2{}, i + 2);
+    if (i + 3 < n) iteration(P3{}, i + 3);
+    if (i + 4 < n) iteration(P4{}, i + 4);
+    if (i + 5 < n) iteration(P5{}, i + 5);
   }
   if (pend_valid) {  // products of the last tile
     bf16x8 pf[2], dsf[2];
@@ -657,8 +693,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       pf[ks] = __builtin_bit_cast(bf16x8, pfw[ks]);
       dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
     }
-    const int last = (n - 1) & 3;
-    compute_dkdv(pf, dsf, s_q[last], s_do[last]);
+    const int last = (n - 1) % NB;
+    compute_dkdv(pf, dsf, s_q[0] + last * TILE_BYTES, s_do[0] + last * TILE_BYTES);
   }
 
   RA_PROF_DUMP;
