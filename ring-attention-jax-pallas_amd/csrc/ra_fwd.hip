@@ -17,6 +17,9 @@
 
 namespace ra {
 
+#ifdef RA_CLOCK
+__device__ unsigned long long g_clock[2];  // timing experiments only: core cycles and 100 MHz ticks of workgroup 0
+#endif
 
 constexpr int kFwdThreads = 512;
 constexpr int kFwdRows = 256;   // query rows per workgroup
@@ -29,10 +32,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   constexpr int DB = D / 32;  // 32-wide blocks of the head dim
   constexpr int TILE_BYTES = kKeyTile * D * 2;
 
-  __shared__ __attribute__((aligned(16))) char s_k[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) char s_v[2][TILE_BYTES];
-  __shared__ __attribute__((aligned(16))) int s_seg[2][kKeyTile];
-  __shared__ __attribute__((aligned(16))) int s_pre[2][kKeyTile];
+  __shared__ __attribute__((aligned(16))) char s_k[4][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) char s_v[4][TILE_BYTES];
+  __shared__ __attribute__((aligned(16))) int s_seg[4][kKeyTile];
+  __shared__ __attribute__((aligned(16))) int s_pre[4][kKeyTile];
   __shared__ unsigned short s_list[GENERAL ? kMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
   __shared__ int s_red[20];
@@ -41,6 +44,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   const int wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
+#ifdef RA_CLOCK
+  // kept in LDS, the kernel has no scalar register to spare
+  __shared__ unsigned long long s_clock[2];
+  if (tid == 0) {
+    s_clock[0] = __builtin_readcyclecounter();
+    s_clock[1] = wall_clock64();
+  }
+#endif
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   int hh, qt;
   decode_block(blockIdx.x, a.B * a.H, nqt, hh, qt);
@@ -71,6 +82,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   const float m_in = a.m[row] * kLog2e;
   float m_run = m_in;  // exponent reference (log2 domain), moves lazily
   float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
+  // Tiles that are completely unmasked add only their ROUNDED probabilities, to this third sum,
+  // which counts for both l and lr: the rounding errors of such a tile's 64 or more terms are
+  // unbiased and their sum moves the logsumexp by far less than its tolerance, and the row sums
+  // cost one dot instruction per pair of scores instead of three additions.
+  float lp_run = 0.f;
   f32x16 oacc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -189,6 +205,17 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       }
     }
   };
+  // one load instruction (RPI rows) of a tile: the loop spreads a tile's instructions over its
+  // MFMA blocks, a burst of them would queue up in the CU's one vector-memory pipe and stall
+  // the issuing waves
+  auto issue_part = [&](const bf16_t* base, const unsigned (&voff)[NLD], long long sl, int k0, unsigned dst, int t) {
+    if (k0 + kKeyTile <= a.Lk) {
+      global_to_lds16_s(base + (long long)(k0 + 8 * wave_u + RPI * t) * sl, voff[t], dst + RPI * t * (D * 2));
+    } else {
+      const int gr = min(k0 + ld_row[t], a.Lk - 1);
+      global_to_lds16(base + (long long)gr * sl + ld_koff[t], dst + RPI * t * (D * 2));
+    }
+  };
   auto issue_k = [&](int j, int buf) {
     const int k0 = j * kKeyTile;
     issue_rows(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + buf * TILE_BYTES + wave_u * 8 * (D * 2));
@@ -201,8 +228,27 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   auto issue_v = [&](int j, int buf) {
     issue_rows(vbase, v_voff, a.v.sl, j * kKeyTile, RA_LDS_ADDR(&s_v[0][0]) + buf * TILE_BYTES + wave_u * 8 * (D * 2));
   };
-  const int n = n_act;
+  const int n = __builtin_amdgcn_readfirstlane(n_act);  // the same in every lane; now the compiler knows
+  j_lo = __builtin_amdgcn_readfirstlane(j_lo);
   int sb_unused;
+  // part t of the request for K tile ordinal j / V tile ordinal j (nothing if the tile does not exist)
+  auto request_k = [&](int j, int t) {
+    if (j < n && t < NLD && !(RA_ABLATE & 1)) {
+      const int k0 = tile_at(j, sb_unused) * kKeyTile;
+      issue_part(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + (j & 3) * TILE_BYTES + wave_u * 8 * (D * 2), t);
+      if (GENERAL && t == 0 && tid < kKeyTile) {
+        int kk = min(k0 + tid, a.Lk - 1);
+        if (kv_seg) seg_r = kv_seg[kk];
+        if (kv_pre) pre_r = kv_pre[kk];
+      }
+    }
+  };
+  auto request_v = [&](int j, int t) {
+    if (j < n && t < NLD && !(RA_ABLATE & 1)) {
+      const int k0 = tile_at(j, sb_unused) * kKeyTile;
+      issue_part(vbase, v_voff, a.v.sl, k0, RA_LDS_ADDR(&s_v[0][0]) + (j & 3) * TILE_BYTES + wave_u * 8 * (D * 2), t);
+    }
+  };
   auto store_ids = [&](int buf) {
     if (GENERAL && tid < kKeyTile) {
       s_seg[buf][tid] = seg_r;
@@ -216,10 +262,19 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   // sum, bf16 packing), and while the 16 MFMAs of O += P(i) V_i run it takes the row maximum of
   // S(i+1).  Vector instructions issued by the wave that owns the MFMA in flight slip into its
   // shadow; the second wave of the SIMD covers LDS and barrier latency.
-  // LDS: K tile j lives in s_k[j & 1], V tile j in s_v[j & 1].  Iteration i reads K_{i+1} and V_i
-  // and, right after the barrier that ends iteration i-1, refills the two buffers nobody reads
-  // any more with K_{i+2} and V_{i+1}.
+  // LDS: K tile j, V tile j and the ids of tile j live in slot j & 3 of their four buffers.
+  // Iteration i reads K_{i+1} (first half: scores of the next tile, probabilities of this one) and
+  // V_i (second half: output update).  Barrier number k publishes K_{k+1} and V_k; right after it
+  // every wave may request its share of K_{k+3} and V_{k+2} (it does so inside its MFMA blocks, one
+  // load instruction at a time): a tile has two iterations to arrive.  Before a barrier a wave
+  // waits until only the requests that follow the previous barrier are in flight.
+  // Waves 0..3 take barrier i at the top of iteration i, waves 4..7 take barrier i+1 BETWEEN the
+  // two halves of iteration i, so that on every SIMD one wave runs its first half (vector-ALU
+  // heavy) and its bookkeeping while the other runs its second half (matrix-unit only).  After
+  // barrier k the tiles K_{k+1}, V_{k-1} (late waves) and V_k are read while K_{k+2}, K_{k+3},
+  // V_{k+1}, V_{k+2} land: three K and four V tiles are live.
   const bool wave_on = qw < a.Lq;
+  // what barriers -3, -2, -1 would have requested
   if (n > 0) {
     issue_k(tile_at(0, sb_unused), 0);
     store_ids(0);
@@ -228,6 +283,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   if (n > 1) {
     issue_k(tile_at(1, sb_unused), 1);
     store_ids(1);
+    issue_v(tile_at(1, sb_unused), 1);
+  }
+  if (n > 2) {
+    issue_k(tile_at(2, sb_unused), 2);
+    store_ids(2);
   }
   __builtin_amdgcn_s_waitcnt(0);  // tiles, carry and Q operands have landed
   __syncthreads();
@@ -353,6 +413,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       m_run = m_new;
       l_run *= corr;
       lr_run *= corr;
+      lp_run *= corr;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -370,6 +431,23 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     plain_lo = max(lo - j_lo, 0);
     plain_hi = min(hi - j_lo, n);
   }
+  plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);  // wave-uniform; now the compiler knows
+  plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
+
+  // Barrier number k and the requests that follow it (see the loop description above).
+  const bool late_half = wave_u >= 4;
+  // second half of iteration i: early waves are between barriers i and i+1 and request V_{i+2},
+  // late waves are between barriers i+1 and i+2 and request V_{i+3}
+  const int v_ahead = late_half ? 3 : 2;
+  auto sync = [&](int k) {
+    // this wave's share of K_{k+1}, V_k is in LDS once only the requests of barrier k-1 (K_{k+2},
+    // V_{k+1}, NLD load instructions each, where they exist) are in flight
+    const int pending = (k + 2 < n ? NLD : 0) + (k + 1 < n ? NLD : 0);
+    if (GENERAL || k == 0 || pending == 0) __builtin_amdgcn_s_waitcnt(0x0f70);
+    else if (pending == NLD) __builtin_amdgcn_s_waitcnt(0x0f70 | NLD);
+    else __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));
+    if (!(RA_ABLATE & 8)) __syncthreads();
+  };
 
   // per-tile state handed from one iteration to the next
   f32x16 sa[2], sb[2];
@@ -388,18 +466,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 
   // one iteration; SC holds S(i) on entry, SN receives S(i+1)
   auto iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
-    constexpr int PAR = decltype(parity)::value;  // i & 1, known at compile time
+    constexpr int PAR = decltype(parity)::value;  // i & 3, known at compile time
     RA_PROF_MARK(i, 1);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of K_{i+1}, V_i is in LDS
-    if (!(RA_ABLATE & 8)) __syncthreads();
+    if (!late_half) sync(i);
     RA_PROF_MARK(i, 2);
-    auto issue_next = [&]() {
-      if (!(RA_ABLATE & 1)) {
-        if (i + 2 < n) issue_k(tile_at(i + 2, sb_unused), PAR);
-        if (i + 1 < n) issue_v(tile_at(i + 1, sb_unused), PAR ^ 1);
-      }
-    };
-    const char* kt = s_k[PAR ^ 1];
+    const char* kt = s_k[(PAR + 1) & 3];
     const char* vt = s_v[PAR];
     int nkt0 = 0, nsegbit = 0, ncls = 1;
     bool nxt_valid = false, nxt_scaled = false;
@@ -413,14 +484,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     float nxt_mx = RA_NEG_INF;
     bf16x8 pfrag[4];
     const bool fused = cur_valid && nxt_valid && !cur_scaled;
-    if (!fused) issue_next();  // the fused path issues the loads inside its second MFMA block
     if (cur_valid) update_reference(cur_mx);
     const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
 
     RA_PROF_MARK(i, 3);
     if (fused) {
       // ---- fused path: S(i+1) MFMAs with the exp2 / sum / pack of tile i in their shadow -------
-      float rs0 = 0.f, rs1 = 0.f;
       {
         bf16x8 fr[2 * KS];
 #pragma unroll
@@ -437,26 +506,32 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
           if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
           if (!(RA_ABLATE & 16)) SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
           else SN[op & 1][op >> 1] += (float)fr[op][0];
+          if (op == (2 * KS) / 4) request_k(i + 3, 0);
+          if (op == (2 * KS) * 3 / 4) request_k(i + 3, 1);
 #pragma unroll
           for (int e = 0; e < ((RA_ABLATE & 2) ? 0 : EPO); e += 2) {
             const int el = op * EPO + e;  // 0..31 over (kb, r)
             const int kb = el >> 4, r = el & 15;
             const float p0 = fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
             const float p1 = fast_exp2(fmaf(SC[kb][r + 1], a.scale2, neg_m));
-            rs0 += p0;
-            rs1 += p1;
             bf16x2 pr;
             pr[0] = (bf16_t)p0;
             pr[1] = (bf16_t)p1;
-            lr_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lr_run, false);
+            // pinned between the two MFMAs: without it the compiler sinks the arithmetic to the
+            // first use of the packed probabilities, behind the MFMA block it is meant to hide in
+            unsigned pw = __builtin_bit_cast(unsigned, pr);
+            asm volatile("" : "+v"(pw));
+            pr = __builtin_bit_cast(bf16x2, pw);
+            lp_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lp_run, false);
+            asm volatile("" : "+v"(lp_run));
             pfrag[2 * kb + (r >> 3)][r & 7] = pr[0];
             pfrag[2 * kb + (r >> 3)][(r & 7) + 1] = pr[1];
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-      l_run += rs0 + rs1;
       RA_PROF_MARK(i, 4);
+      if (late_half) sync(i + 1);
       // ---- O += P(i) V_i with the row maximum of S(i+1) in the shadow ---------------------------
       {
         bf16x8 fr[4 * DB];
@@ -470,12 +545,13 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
           if (op + PF < 4 * DB) fr[op + PF] = pv_op_frag(vt, op + PF);
           if (!(RA_ABLATE & 4)) oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
           else oacc[op % DB][op / DB] += (float)fr[op][0] * (float)pfrag[op / DB][0];
-          if (op == 1) issue_next();  // direct-to-LDS loads of K_{i+2}, V_{i+1}: issue cost hidden behind the MFMAs
+          if (op == (4 * DB) / 4) request_v(i + v_ahead, 0);
+          if (op == (4 * DB) * 3 / 4) request_v(i + v_ahead, 1);
 #pragma unroll
           for (int e = 0; e < EPO; e += 2) {
-            const int el = op * EPO + e;
-            mx0 = fmaxf(mx0, SN[el >> 4][el & 15]);
-            mx1 = fmaxf(mx1, SN[el >> 4][(el & 15) + 1]);
+            const int el = op * EPO + e;  // one three-operand maximum per pair of scores
+            float& mx = (op & 1) ? mx1 : mx0;
+            mx = fmaxf(fmaxf(mx, SN[el >> 4][el & 15]), SN[el >> 4][(el & 15) + 1]);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -484,6 +560,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       RA_PROF_MARK(i, 5);
     } else {
       // ---- generic path (first / last / masked / biased tiles): same work, not interleaved -----
+      request_k(i + 3, 0);
+      request_k(i + 3, 1);
       if (nxt_valid) compute_s(SN, kt);
       if (cur_valid) {
         float rs = 0.f;
@@ -509,29 +587,204 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
               lr_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lr_run, false);
             }
           }
-        compute_pv(pfrag, vt);
       }
+      if (late_half) sync(i + 1);
+      request_v(i + v_ahead, 0);
+      request_v(i + v_ahead, 1);
+      if (cur_valid) compute_pv(pfrag, vt);
       if (nxt_valid && !nxt_scaled) nxt_mx = raw_rowmax(SN);
     }
     RA_PROF_MARK(i, 6);
-    if (nxt_scaled) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, PAR ^ 1);
-    if (i + 2 < n) store_ids(PAR);
+    if (nxt_scaled) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, (i + 1) & 3);
+    if (i + 3 < n) store_ids((i + 3) & 3);
     cur_valid = nxt_valid;
     cur_scaled = nxt_scaled;
     cur_mx = nxt_mx;
   };
 
-  for (int i = 0; i < n; i += 2) {
-    iteration(std::integral_constant<int, 0>{}, i, sa, sb);
-    if (i + 1 < n) iteration(std::integral_constant<int, 1>{}, i + 1, sb, sa);
+  // ---- the same iteration for a stretch of plain tiles ---------------------------------------------
+  // Tiles i and i+1 are seen completely, unmasked and in range by this wave, and the tiles that the
+  // iteration requests (K_{i+3}; V_{i+2} for the early waves, V_{i+3} for the late ones) exist and
+  // are complete: straight-line code, no classification, no flags, scalar running addresses.
+  const bf16_t* k_run = kbase;
+  const bf16_t* v_run = vbase;
+  const long long k_part = (long long)RPI * a.k.sl, v_part = (long long)RPI * a.v.sl;
+  const unsigned k_dst0 = RA_LDS_ADDR(&s_k[0][0]) + wave_u * 8 * (D * 2);
+  const unsigned v_dst0 = RA_LDS_ADDR(&s_v[0][0]) + wave_u * 8 * (D * 2);
+  auto seek_plain = [&](int ordinal) {  // the iteration with this ordinal is the next to run
+    k_run = kbase + (long long)((j_lo + ordinal + 3) * kKeyTile + 8 * wave_u) * a.k.sl;
+    v_run = vbase + (long long)((j_lo + ordinal + v_ahead) * kKeyTile + 8 * wave_u) * a.v.sl;
+  };
+  auto sync_plain = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));  // only the previous barrier's requests are in flight
+    __syncthreads();
+  };
+  auto plain_iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
+    constexpr int PAR = decltype(parity)::value;
+    RA_PROF_MARK(i, 1);
+    if (!late_half) sync_plain();
+    RA_PROF_MARK(i, 2);
+    const char* kt = s_k[(PAR + 1) & 3];
+    const char* vt = s_v[PAR];
+    update_reference(cur_mx);
+    const float neg_m = -m_run;  // finite: the current tile has unmasked scores
+    const unsigned v_dst = v_dst0 + (late_half ? ((PAR + 3) & 3) : ((PAR + 2) & 3)) * TILE_BYTES;
+    RA_PROF_MARK(i, 3);
+    // ---- S(i+1) MFMAs, then O += P(i) V_i, with the softmax arithmetic of tile i and the row
+    // maximum of S(i+1) in their shadow.  The chain of a pair of scores (scale and shift, exp2,
+    // pack, row sum) is spread over four consecutive MFMA slots, one link per slot, so that no
+    // vector instruction waits for the result of the one before it; the sixteen pairs of a lane
+    // are spread over both MFMA blocks so that every slot carries about the same vector work:
+    // half of them (the first two operand fragments of P) in the score block, the other half in
+    // the first three quarters of the output block, the row maxima in the slots that remain.
+    constexpr int NOPA = 2 * KS, NOPB = 4 * DB;
+    auto slot_of = [](int w) constexpr -> int {  // global slot (score block first) of pair w's exp2
+      if (D == 128) return w < 8 ? 2 * w : 16 + (3 * (w - 8)) / 2;
+      return w < 8 ? w : 8 + (w - 8) / 2;
+    };
+    auto maxima_in = [](int sb) constexpr -> int {  // row-maximum instructions in slot sb of the output block
+      if (D == 128) return (sb >= 12 || sb % 3 == 2) ? 2 : 0;
+      return 2;
+    };
+    float t[16][2], e[16][2];
+    unsigned pk[16];
+    u32x4 pw[4];
+    auto link1 = [&](int w) {  // pair w = elements 2w, 2w+1 of the 32 scores of this lane
+      const int kb = (2 * w) >> 4, r = (2 * w) & 15;
+      t[w][0] = fmaf(SC[kb][r], a.scale2, neg_m);
+      t[w][1] = fmaf(SC[kb][r + 1], a.scale2, neg_m);
+      asm volatile("" : "+v"(t[w][0]), "+v"(t[w][1]));
+    };
+    auto link2 = [&](int w) {
+      e[w][0] = fast_exp2(t[w][0]);
+      e[w][1] = fast_exp2(t[w][1]);
+      asm volatile("" : "+v"(e[w][0]), "+v"(e[w][1]));
+    };
+    auto link3 = [&](int w) {
+      bf16x2 pr;
+      pr[0] = (bf16_t)e[w][0];
+      pr[1] = (bf16_t)e[w][1];
+      pk[w] = __builtin_bit_cast(unsigned, pr);
+      asm volatile("" : "+v"(pk[w]));
+      pw[w >> 2][w & 3] = pk[w];
+    };
+    auto link4 = [&](int w) {
+      lp_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lp_run, false);
+      asm volatile("" : "+v"(lp_run));
+    };
+    auto links_of_slot = [&](int gs) {
+#pragma unroll
+      for (int w = 0; w < 16; ++w) {
+        if (slot_of(w) - 1 == gs) link1(w);
+        if (slot_of(w) == gs) link2(w);
+        if (slot_of(w) + 1 == gs) link3(w);
+        if (slot_of(w) + 2 == gs) link4(w);
+      }
+    };
+    {
+      bf16x8 fr[NOPA];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        SN[0][r] = 0.f;
+        SN[1][r] = 0.f;
+      }
+#pragma unroll
+      for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
+      links_of_slot(-1);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int op = 0; op < NOPA; ++op) {
+        if (op + PF < NOPA) fr[op + PF] = s_op_frag(kt, op + PF);
+        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
+        if (op == NOPA / 4) global_to_lds16_s(k_run, k_voff[0], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES);
+        if (NLD == 2 && op == NOPA * 3 / 4)
+          global_to_lds16_s(k_run + k_part, k_voff[NLD - 1], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES + RPI * (D * 2));
+        links_of_slot(op);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    k_run += (long long)kKeyTile * a.k.sl;
+    RA_PROF_MARK(i, 4);
+    if (late_half) sync_plain();
+    {
+      bf16x8 fr[NOPB];
+      float mx0 = RA_NEG_INF, mx1 = RA_NEG_INF;
+#pragma unroll
+      for (int op = 0; op < PF; ++op) fr[op] = pv_op_frag(vt, op);
+      __builtin_amdgcn_sched_barrier(0);
+      int el = 0;  // next pair of S(i+1) elements to enter the row maximum
+#pragma unroll
+      for (int op = 0; op < NOPB; ++op) {
+        if (op + PF < NOPB) fr[op + PF] = pv_op_frag(vt, op + PF);
+        oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            fr[op], __builtin_bit_cast(bf16x8, pw[op / DB]), oacc[op % DB], 0, 0, 0);
+        if (op == NOPB / 4) global_to_lds16_s(v_run, v_voff[0], v_dst);
+        if (NLD == 2 && op == NOPB * 3 / 4) global_to_lds16_s(v_run + v_part, v_voff[NLD - 1], v_dst + RPI * (D * 2));
+        links_of_slot(NOPA + op);
+#pragma unroll
+        for (int x = 0; x < maxima_in(op); ++x) {
+          float& mx = (x & 1) ? mx1 : mx0;  // one three-operand maximum per pair of scores
+          mx = fmaxf(fmaxf(mx, SN[el >> 4][el & 15]), SN[el >> 4][(el & 15) + 1]);
+          asm volatile("" : "+v"(mx));
+          el += 2;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      cur_mx = half_max(fmaxf(mx0, mx1)) * a.scale2;
+    }
+    v_run += (long long)kKeyTile * a.v.sl;
+    RA_PROF_MARK(i, 5);
+  };
+
+  if (late_half) {
+    sync(0);
+    request_v(2, 0);  // what the second half of iteration -1 would have requested
+    request_v(2, 1);
   }
+  // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
+  // plain stretch in whole groups of four, generic iterations for the rest.  Every wave runs n
+  // iterations in total, so the barrier counts agree.
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  using P2 = std::integral_constant<int, 2>;
+  using P3 = std::integral_constant<int, 3>;
+  // iteration i is plain for plain_lo <= i < plain_end
+  const int plain_end =
+      __builtin_amdgcn_readfirstlane(use_list ? 0 : min(min(plain_hi - 1, n - 3), a.Lk / kKeyTile - j_lo - 3));
+  int i = 0;
+  for (; i < n && !(i >= plain_lo && i + 4 <= plain_end); i += 4) {
+    iteration(P0{}, i, sa, sb);
+    if (i + 1 < n) iteration(P1{}, i + 1, sb, sa);
+    if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
+    if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
+  }
+  if (i + 4 <= plain_end) seek_plain(i);
+  for (; i + 4 <= plain_end; i += 4) {
+    plain_iteration(P0{}, i, sa, sb);
+    plain_iteration(P1{}, i + 1, sb, sa);
+    plain_iteration(P2{}, i + 2, sa, sb);
+    plain_iteration(P3{}, i + 3, sb, sa);
+  }
+  for (; i < n; i += 4) {
+    iteration(P0{}, i, sa, sb);
+    if (i + 1 < n) iteration(P1{}, i + 1, sb, sa);
+    if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
+    if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
+  }
+  if (!late_half) sync(n);  // both halves pass the same number of barriers
 
   RA_PROF_DUMP;
+#ifdef RA_CLOCK
+  if (blockIdx.x == 0 && tid == 0) {
+    g_clock[0] = __builtin_readcyclecounter() - s_clock[0];
+    g_clock[1] = wall_clock64() - s_clock[1];
+  }
+#endif
   // ---- merge this step into the carry ---------------------------------------------------------
   // o = o_in 2^(m_in - m_out) + o_step 2^(m_run - m_out) l_step / lr_step,  l likewise with the
   // exact sum, m_out = exact maximum over carry and step.
   {
-    const float l_step = half_sum(l_run), lr_step = half_sum(lr_run);
+    const float l_step = half_sum(l_run + lp_run), lr_step = half_sum(lr_run + lp_run);
     const float m_out = m_true;  // started from m_in, so it already covers the carry
     const float m_safe = (m_out == RA_NEG_INF) ? 0.f : m_out;
     const float f_in = fast_exp2(m_in - m_safe);   // 0 for an empty carry
