@@ -25,6 +25,7 @@ constexpr int kFwdThreads = 512;
 constexpr int kFwdRows = 256;   // query rows per workgroup
 constexpr int kKeyTile = 64;    // keys per LDS tile
 constexpr int kMaxListTiles = 1024;
+constexpr int kPlainMinTiles = 16;  // shortest stretch of plain tiles that takes the straight-line loop
 
 template <int D, bool GENERAL>
 __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) {
@@ -82,10 +83,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   const float m_in = a.m[row] * kLog2e;
   float m_run = m_in;  // exponent reference (log2 domain), moves lazily
   float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
-  // Tiles that are completely unmasked add only their ROUNDED probabilities, to this third sum,
-  // which counts for both l and lr: the rounding errors of such a tile's 64 or more terms are
-  // unbiased and their sum moves the logsumexp by far less than its tolerance, and the row sums
-  // cost one dot instruction per pair of scores instead of three additions.
+  // In a long stretch of completely unmasked tiles (at least kPlainMinTiles of them) a tile adds
+  // only its ROUNDED probabilities, to this third sum, which counts for both l and lr: the
+  // rounding errors of the thousand or more terms are unbiased and their sum moves the logsumexp
+  // by a few 1e-5, far less than its tolerance, and the row sums cost one dot instruction per
+  // pair of scores instead of three additions.
   float lp_run = 0.f;
   f32x16 oacc[DB];
 #pragma unroll
@@ -490,6 +492,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     RA_PROF_MARK(i, 3);
     if (fused) {
       // ---- fused path: S(i+1) MFMAs with the exp2 / sum / pack of tile i in their shadow -------
+      float rs0 = 0.f, rs1 = 0.f;
       {
         bf16x8 fr[2 * KS];
 #pragma unroll
@@ -514,6 +517,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
             const int kb = el >> 4, r = el & 15;
             const float p0 = fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
             const float p1 = fast_exp2(fmaf(SC[kb][r + 1], a.scale2, neg_m));
+            rs0 += p0;
+            rs1 += p1;
             bf16x2 pr;
             pr[0] = (bf16_t)p0;
             pr[1] = (bf16_t)p1;
@@ -522,14 +527,15 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
             unsigned pw = __builtin_bit_cast(unsigned, pr);
             asm volatile("" : "+v"(pw));
             pr = __builtin_bit_cast(bf16x2, pw);
-            lp_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lp_run, false);
-            asm volatile("" : "+v"(lp_run));
+            lr_run = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, lr_run, false);
+            asm volatile("" : "+v"(lr_run));
             pfrag[2 * kb + (r >> 3)][r & 7] = pr[0];
             pfrag[2 * kb + (r >> 3)][(r & 7) + 1] = pr[1];
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
+      l_run += rs0 + rs1;
       RA_PROF_MARK(i, 4);
       if (late_half) sync(i + 1);
       // ---- O += P(i) V_i with the row maximum of S(i+1) in the shadow ---------------------------
@@ -750,7 +756,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   using P3 = std::integral_constant<int, 3>;
   // iteration i is plain for plain_lo <= i < plain_end
   const int plain_end =
-      __builtin_amdgcn_readfirstlane(use_list ? 0 : min(min(plain_hi - 1, n - 3), a.Lk / kKeyTile - j_lo - 3));
+      __builtin_amdgcn_readfirstlane((use_list || plain_hi - plain_lo < kPlainMinTiles)
+                                         ? 0
+                                         : min(min(plain_hi - 1, n - 3), a.Lk / kKeyTile - j_lo - 3));
   int i = 0;
   for (; i < n && !(i >= plain_lo && i + 4 <= plain_end); i += 4) {
     iteration(P0{}, i, sa, sb);
