@@ -93,6 +93,30 @@ class EventTimer:
         return [(key, a.elapsed_time(b)) for key, a, b in self.records]
 
 
+def mfma_ceiling(torch, dev):
+    """bf16 MFMA rate of a loop of nothing but v_mfma_f32_32x32x16_bf16 with operands that toggle
+    like real data, one wave per SIMD on every compute unit, ~15 ms per launch: what the board's
+    power management leaves of the published peak.  Reported next to `roofline`, never used in it."""
+    import ctypes as C
+    from ring_attention import _lib
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    iters = 100000
+    sink = torch.empty(cus * 256, device=dev, dtype=torch.float32)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    best = 0.0
+    for rep in range(4):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record(torch.cuda.current_stream())
+        _lib.check("ra_probe_mfma_rate", lib.ra_probe_mfma_rate(sink.data_ptr(), cus, iters, 1, stream))
+        b.record(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        if rep:  # the first launch runs while the clock is still ramping
+            best = max(best, cus * 4 * iters * 8 * 32768.0 / (a.elapsed_time(b) * 1e-3) / 1e12)
+    return {"value": round(best, 1), "unit": "TFLOP/s", "frac_of_published_peak": round(best / PEAK_BF16_TFLOPS, 4),
+            "what": "v_mfma_f32_32x32x16_bf16 only, random operands in registers, one wave per SIMD, all CUs"}
+
+
 def cpu_baseline(D):
     """The numpy restatement of the reference algorithm, timed on the host cores on a bounded
     sample of the workload (same head dim, causal, fp32): H=8, S=16384 as 4 shards of 4096."""
@@ -280,6 +304,9 @@ def main():
             P7 = sum(pairs[(n - 1, ks)] for ks in range(n))
             result["rank7_share"] = {"fwd_tflops": round(4.0 * D * P7 * B * H / f_ms / 1e9, 2),
                                      "bwd_tflops": round(10.0 * D * P7 * B * H / b_ms / 1e9, 2)}
+
+    if not args.no_kernel_timing:
+        result["mfma_ceiling"] = mfma_ceiling(torch, dev)
 
     if args.copy_probe:
         # a kernel of known traffic (reads 1 GiB, writes 1 GiB) for scaling profiler byte counters

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(CSRC, "build")
 LIB_PATH = os.path.join(HERE, "ring_attention", "libringattn_hip.so")
-SOURCES = ["ra_fwd.hip", "ra_bwd.hip", "ra_api.hip"]
+SOURCES = ["ra_fwd.hip", "ra_bwd.hip", "ra_api.hip", "ra_probe.hip"]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

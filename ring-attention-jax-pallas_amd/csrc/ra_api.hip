@@ -248,4 +248,12 @@ int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t o
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_finalize launch");
 }
 
+int ra_probe_mfma_rate(float* sink, int32_t blocks, int32_t iters, int32_t random_operands, void* stream) {
+  if (!sink) return fail(RA_ERR_NULL, "ra_probe_mfma_rate: sink is NULL");
+  if (blocks <= 0 || blocks > 65536 || iters <= 0 || (iters % 4))
+    return fail(RA_ERR_SHAPE, "ra_probe_mfma_rate: blocks in [1, 65536], iters a positive multiple of 4");
+  hipError_t e = ra::launch_mfma_rate(sink, blocks, iters, random_operands != 0, (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_probe_mfma_rate launch");
+}
+
 }  // extern "C"

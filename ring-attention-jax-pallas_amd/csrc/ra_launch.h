@@ -37,6 +37,7 @@ hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long lon
                             TensorArg dout, float* delta, int B, int H, int Lq, int D,
                             hipStream_t stream);
 hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, int parts, hipStream_t stream);
+hipError_t launch_mfma_rate(float* sink, int blocks, int iters, int random, hipStream_t stream);
 hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl,
                                int B, int H, int L, int D, hipStream_t stream);
 
