@@ -137,6 +137,31 @@ def test_sorted_segments_and_alibi(device):
            R.make_bias_fn(causal=True, alibi=sl))
 
 
+def test_fully_masked_rows_do_not_poison_key_gradients(device):
+    # queries whose segment id matches no key: o = NaN, lse = -inf like the reference
+    # (ring.py:134-135); such rows must contribute nothing to dk / dv.  The expected gradients
+    # are those of the attention restricted to the queries that do see a key.
+    print("[parity] fully masked rows: dk / dv stay finite", flush=True)
+    B, S, H, D, n = 1, 512, 2, 128, 4
+    q, k, v, do = R.make_inputs(11, B, S, S, H, D)
+    rng = np.random.default_rng(11)
+    ks = rng.integers(0, 3, (B, S)).astype(np.int32)
+    qs = rng.integers(0, 4, (B, S)).astype(np.int32)  # id 3 matches no key
+    out, lse, g = _run_hip(device, q, k, v, do, n, ra.segment_bias(), {"q_segment_ids": qs},
+                           {"kv_segment_ids": ks})
+    dead = qs[0] == 3
+    assert dead.any() and not dead.all()
+    assert np.isnan(out[0, dead]).all() and np.isneginf(lse[0][:, dead]).all()
+    live = ~dead
+    bias = R.make_bias_fn(use_segments=True)(q_segment_ids=qs[:, live], kv_segment_ids=ks)
+    wq, wk, wv = R.mha_dense_grads(q[:, live], k, v, do[:, live], bias)
+    dq, dk, dv = g
+    assert np.isfinite(dk).all() and np.isfinite(dv).all()
+    for got, ref, nm in ((dq[:, live], wq, "dq"), (dk, wk, "dk"), (dv, wv, "dv")):
+        mx, fro = _rel(got, ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+
+
 def test_prefix_lm(device):
     pm = (np.arange(512)[None, :] < np.array([[100], [300]])).astype(np.int32)
     _check(device, "prefix", 2, 512, 512, 2, 64, 4, ra.prefix_lm_bias(), R.make_bias_fn(use_prefix=True),
