@@ -659,7 +659,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
   // iteration i is plain for plain_lo < i < plain_end (tile i+3 must exist and be complete)
-  const int plain_end = min(min(plain_hi - 1, n - 3), a.Lq / kQTile - i_lo - 3);
+  const int plain_end = GENERAL ? -1 : min(min(plain_hi - 1, n - 3), a.Lq / kQTile - i_lo - 3);
   int i = 0;
   for (; i < n && !(i > plain_lo && i + NB <= plain_end); i += NB) {
     iteration(P0{}, i);
@@ -669,14 +669,16 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (i + 4 < n) iteration(P4{}, i + 4);
     if (i + 5 < n) iteration(P5{}, i + 5);
   }
-  if (i + NB <= plain_end) seek_plain(i_lo + i + 3);
-  for (; i + NB <= plain_end; i += NB) {
-    plain_iteration(P0{}, i);
-    plain_iteration(P1{}, i + 1);
-    plain_iteration(P2{}, i + 2);
-    plain_iteration(P3{}, i + 3);
-    plain_iteration(P4{}, i + 4);
-    plain_iteration(P5{}, i + 5);
+  if constexpr (!GENERAL) {  // the GENERAL variants are launched for biases that leave no plain stretch
+    if (i + NB <= plain_end) seek_plain(i_lo + i + 3);
+    for (; i + NB <= plain_end; i += NB) {
+      plain_iteration(P0{}, i);
+      plain_iteration(P1{}, i + 1);
+      plain_iteration(P2{}, i + 2);
+      plain_iteration(P3{}, i + 3);
+      plain_iteration(P4{}, i + 4);
+      plain_iteration(P5{}, i + 5);
+    }
   }
   for (; i < n; i += NB) {
     iteration(P0{}, i);
@@ -1173,7 +1175,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   using P3 = std::integral_constant<int, 3>;
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
-  const int plain_end = min(plain_hi - 1, n - 3);  // iteration i is plain for plain_lo < i < plain_end
+  const int plain_end = GENERAL ? -1 : min(plain_hi - 1, n - 3);  // iteration i is plain for plain_lo < i < plain_end
   int i = 0;
   for (; i < n && !(i > plain_lo && i + 6 <= plain_end); i += 6) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
@@ -1183,13 +1185,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  for (; i + 6 <= plain_end; i += 6) {
-    plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
-    plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
-    plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
-    plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
-    plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
-    plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+  if constexpr (!GENERAL) {  // the GENERAL variants are launched for biases that leave no plain stretch
+    for (; i + 6 <= plain_end; i += 6) {
+      plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
+      plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+      plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+      plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+      plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+      plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+    }
   }
   for (; i < n; i += 6) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
   }
-  const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
+  long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
   // This step accumulates its own contribution from zero and is merged with the incoming carry
   // at the end.  Two row sums are kept: l_run adds the fp32 probabilities (it becomes the
   // carry's l and the logsumexp), lr_run adds the SAME probabilities after their rounding to
@@ -80,8 +80,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   // l_run / lr_run makes it a properly normalised average of V times the exact row sum, so
   // the rounding of P cancels in o / l instead of showing up as an error of order 2^-9 |v|
   // on rows that see only a few keys.
-  const float m_in = a.m[row] * kLog2e;
-  float m_run = m_in;  // exponent reference (log2 domain), moves lazily
+  float m_run = a.m[row] * kLog2e;  // exponent reference (log2 domain), moves lazily
   float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
   // In a long stretch of completely unmasked tiles (at least kPlainMinTiles of them) a tile adds
   // only its ROUNDED probabilities, to this third sum, which counts for both l and lr: the
@@ -182,15 +181,19 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   constexpr int CPR = D / 8;            // 16-byte chunks per row
   constexpr int RPI = 64 / CPR;         // rows per load instruction
   constexpr int NLD = 8 / RPI;          // load instructions per wave per tile
-  int ld_row[NLD], ld_koff[NLD];
   unsigned k_voff[NLD], v_voff[NLD];  // per-lane byte offsets inside a group of RPI rows
+  // row inside the tile and element offset of the chunk that a lane moves with instruction t
+  // (recomputed where the rare partial-tile path needs them: registers are scarce here)
+  auto ld_row = [&](int t) { return 8 * wave + RPI * t + lane / CPR; };
+  auto ld_koff = [&](int t) {
+    const int rrow = 8 * wave + RPI * t + lane / CPR;
+    return ((tile_off<D>(rrow, lane % CPR) - rrow * (D * 2)) >> 4) * 8;
+  };
 #pragma unroll
   for (int t = 0; t < NLD; ++t) {
     const int rrow = 8 * wave + RPI * t + lane / CPR;
     const int pc = lane % CPR;
     const int lc = (tile_off<D>(rrow, pc) - rrow * (D * 2)) >> 4;  // logical chunk stored at pc
-    ld_row[t] = rrow;
-    ld_koff[t] = lc * 8;
     k_voff[t] = (unsigned)(((long long)(lane / CPR) * a.k.sl + lc * 8) * 2);
     v_voff[t] = (unsigned)(((long long)(lane / CPR) * a.v.sl + lc * 8) * 2);
   }
@@ -202,8 +205,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     } else {  // last, partial tile: rows past the end repeat the last row (masked later)
 #pragma unroll
       for (int t = 0; t < NLD; ++t) {
-        const int gr = min(k0 + ld_row[t], a.Lk - 1);
-        global_to_lds16(base + (long long)gr * sl + ld_koff[t], dst + RPI * t * (D * 2));
+        const int gr = min(k0 + ld_row(t), a.Lk - 1);
+        global_to_lds16(base + (long long)gr * sl + ld_koff(t), dst + RPI * t * (D * 2));
       }
     }
   };
@@ -214,8 +217,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (k0 + kKeyTile <= a.Lk) {
       global_to_lds16_s(base + (long long)(k0 + 8 * wave_u + RPI * t) * sl, voff[t], dst + RPI * t * (D * 2));
     } else {
-      const int gr = min(k0 + ld_row[t], a.Lk - 1);
-      global_to_lds16(base + (long long)gr * sl + ld_koff[t], dst + RPI * t * (D * 2));
+      const int gr = min(k0 + ld_row(t), a.Lk - 1);
+      global_to_lds16(base + (long long)gr * sl + ld_koff(t), dst + RPI * t * (D * 2));
     }
   };
   auto issue_k = [&](int j, int buf) {
@@ -319,18 +322,23 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       const int j = lane & 15;
       const int vrow = 4 * g + (j >> 2) + 8 * hh2;
       const int vcol = 32 * db + 16 * ((lane >> 4) & 1) + 4 * (j & 3);
-      voff[db][hh2] = tile_off<D>(vrow, vcol >> 3) + ((vcol & 4) << 1);
+      // The V buffers start beyond the 64 KiB that an LDS instruction's immediate offset can span:
+      // their base is part of the per-lane address (made opaque, so that the compiler does not
+      // fold it back into the immediate and re-add it with a vector instruction per fetch).
+      unsigned va = RA_LDS_ADDR(&s_v[0][0]) + tile_off<D>(vrow, vcol >> 3) + ((vcol & 4) << 1);
+      asm volatile("" : "+v"(va));
+      voff[db][hh2] = (int)va;
     }
   constexpr int ROWB = D * 2;
   auto s_op_frag = [&](const char* kt, int op) {
     if (RA_ABLATE & 32) return qf[op >> 1];
     return *(const bf16x8*)(kt + (32 * (op & 1)) * ROWB + koff[op >> 1]);
   };
-  auto pv_op_frag = [&](const char* vt, int op) {
+  auto pv_op_frag = [&](unsigned vt, int op) {  // vt: byte offset of the tile buffer inside s_v
     if (RA_ABLATE & 64) return qf[op % KS];
-    const int cofs = (32 * (op / (2 * DB)) + 16 * ((op / DB) & 1)) * ROWB;
-    const lds_char* p0 = (const lds_char*)(vt + cofs + voff[op % DB][0]);
-    const lds_char* p1 = (const lds_char*)(vt + cofs + voff[op % DB][1]);
+    const unsigned cofs = (32 * (op / (2 * DB)) + 16 * ((op / DB) & 1)) * ROWB;
+    const lds_char* p0 = (const lds_char*)(uintptr_t)((unsigned)voff[op % DB][0] + (vt + cofs));
+    const lds_char* p1 = (const lds_char*)(uintptr_t)((unsigned)voff[op % DB][1] + (vt + cofs));
     bf16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p0);
     bf16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)p1);
     return __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -353,7 +361,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  auto compute_pv = [&](const bf16x8 (&pf)[4], const char* vt) {
+  auto compute_pv = [&](const bf16x8 (&pf)[4], unsigned vt) {
     bf16x8 fr[4 * DB];
 #pragma unroll
     for (int op = 0; op < PF; ++op) fr[op] = pv_op_frag(vt, op);
@@ -473,7 +481,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (!late_half) sync(i);
     RA_PROF_MARK(i, 2);
     const char* kt = s_k[(PAR + 1) & 3];
-    const char* vt = s_v[PAR];
+    const unsigned vt = PAR * TILE_BYTES;
     int nkt0 = 0, nsegbit = 0, ncls = 1;
     bool nxt_valid = false, nxt_scaled = false;
     if (i + 1 >= plain_lo && i + 1 < plain_hi) {
@@ -631,7 +639,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (!late_half) sync_plain();
     RA_PROF_MARK(i, 2);
     const char* kt = s_k[(PAR + 1) & 3];
-    const char* vt = s_v[PAR];
+    const unsigned vt = PAR * TILE_BYTES;
     update_reference(cur_mx);
     const float neg_m = -m_run;  // finite: the current tile has unmasked scores
     const unsigned v_dst = v_dst0 + (late_half ? ((PAR + 3) & 3) : ((PAR + 2) & 3)) * TILE_BYTES;
@@ -756,7 +764,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   using P3 = std::integral_constant<int, 3>;
   // iteration i is plain for plain_lo <= i < plain_end
   const int plain_end =
-      __builtin_amdgcn_readfirstlane((use_list || plain_hi - plain_lo < kPlainMinTiles)
+      __builtin_amdgcn_readfirstlane((GENERAL || use_list || plain_hi - plain_lo < kPlainMinTiles)
                                          ? 0
                                          : min(min(plain_hi - 1, n - 3), a.Lk / kKeyTile - j_lo - 3));
   int i = 0;
@@ -766,12 +774,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
     if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
   }
-  if (i + 4 <= plain_end) seek_plain(i);
-  for (; i + 4 <= plain_end; i += 4) {
-    plain_iteration(P0{}, i, sa, sb);
-    plain_iteration(P1{}, i + 1, sb, sa);
-    plain_iteration(P2{}, i + 2, sa, sb);
-    plain_iteration(P3{}, i + 3, sb, sa);
+  if constexpr (!GENERAL) {  // the GENERAL variants are launched for biases that leave no plain stretch
+    if (i + 4 <= plain_end) seek_plain(i);
+    for (; i + 4 <= plain_end; i += 4) {
+      plain_iteration(P0{}, i, sa, sb);
+      plain_iteration(P1{}, i + 1, sb, sa);
+      plain_iteration(P2{}, i + 2, sa, sb);
+      plain_iteration(P3{}, i + 3, sb, sa);
+    }
   }
   for (; i < n; i += 4) {
     iteration(P0{}, i, sa, sb);
@@ -792,6 +802,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   // o = o_in 2^(m_in - m_out) + o_step 2^(m_run - m_out) l_step / lr_step,  l likewise with the
   // exact sum, m_out = exact maximum over carry and step.
   {
+    // the row index and the incoming maximum are recomputed / reloaded: not worth two registers
+    // over the whole loop
+    row = ((long long)b * a.H + h) * a.Lq + min(q0 + wave * 32 + l32, a.Lq - 1);
+    const float m_in = a.m[row] * kLog2e;
     const float l_step = half_sum(l_run + lp_run), lr_step = half_sum(lr_run + lp_run);
     const float m_out = m_true;  // started from m_in, so it already covers the carry
     const float m_safe = (m_out == RA_NEG_INF) ? 0.f : m_out;
