@@ -326,6 +326,35 @@ RA_DEV void query_tile_range(int flags, int window, int klo, int khi, int q_off,
   lo = min(max(lo, 0), hi);
 }
 
+// Executed by ONE wave.  `list` holds `cnt` entries (tile index in bits 0..14, bit 15 set when
+// the tile needs the elementwise segment test).  Finds the first run of entries that need no test
+// and whose tile indices are consecutive: ordinals [start, end), and `tile_base` such that entry
+// i of the run is tile `tile_base + i`.  Such a run can be walked with running addresses.
+RA_DEV void uniform_run(const unsigned short* list, int cnt, int lane, int& start, int& end, int& tile_base) {
+  start = -1;
+  for (int base = 0; base < cnt && start < 0; base += 64) {
+    const int i = base + lane;
+    const bool ok = i < cnt && !(list[i] >> 15);
+    const unsigned long long mask = __ballot(ok);
+    if (mask) start = base + __ffsll((long long)mask) - 1;
+  }
+  if (start < 0) {
+    start = end = tile_base = 0;
+    return;
+  }
+  end = cnt;
+  for (int base = start; base < cnt; base += 64) {
+    const int i = base + lane;
+    const bool brk = i < cnt && i > start && ((list[i] >> 15) || (list[i] & 0x7fff) != (list[i - 1] & 0x7fff) + 1);
+    const unsigned long long mask = __ballot(brk);
+    if (mask) {
+      end = base + __ffsll((long long)mask) - 1;
+      break;
+    }
+  }
+  tile_base = (list[start] & 0x7fff) - start;
+}
+
 // Decode the flat workgroup id into (batch*head index, tile index).  Workgroups are handed
 // to the 8 XCDs round-robin, each XCD has its own L2: keep all tiles of one head on one
 // XCD so they share the head's K/V (or Q/dO) stream, and start with the last tile, which

@@ -39,7 +39,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   __shared__ __attribute__((aligned(16))) int s_pre[4][kKeyTile];
   __shared__ unsigned short s_list[GENERAL ? kMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
-  __shared__ int s_red[20];
+  __shared__ int s_red[24];
+  __shared__ int s_stash[GENERAL ? 3 : 1][GENERAL ? kFwdThreads : 1];
+  // The GENERAL variant is four registers short in its straight-line loop: the first operand
+  // fragment of Q waits here and is fetched once per iteration instead.
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q0[GENERAL ? kFwdThreads : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -71,6 +75,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     const bf16_t* qp = a.q.ptr + b * a.q.sb + h * a.q.sh + (long long)qi_c * a.q.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
+    if (GENERAL) s_q0[tid] = qf[0];
   }
   long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
   // This step accumulates its own contribution from zero and is merged with the incoming carry
@@ -114,6 +119,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
+  // ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` that need no segment test
+  int run_lo = 0, run_hi = n_act, tile_base = j_lo;
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     // segment-id range of the workgroup's queries, then one thread per key tile decides
     // whether the id ranges can intersect (skip otherwise) and whether the tile is uniform
@@ -154,10 +161,20 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
         if (f) s_list[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)((j_lo + i) | ((f & 2) << 14));
         cnt += __popcll(mask);
       }
-      if (lane == 0) s_red[16] = cnt;
+      int u_lo, u_hi, u_base;
+      uniform_run(s_list, cnt, lane, u_lo, u_hi, u_base);
+      if (lane == 0) {
+        s_red[16] = cnt;
+        s_red[17] = u_lo;
+        s_red[18] = u_hi;
+        s_red[19] = u_base;
+      }
     }
     __syncthreads();
     n_act = s_red[16];
+    run_lo = s_red[17];
+    run_hi = s_red[18];
+    tile_base = s_red[19];
   }
 
   const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
@@ -235,6 +252,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   };
   const int n = __builtin_amdgcn_readfirstlane(n_act);  // the same in every lane; now the compiler knows
   j_lo = __builtin_amdgcn_readfirstlane(j_lo);
+  run_lo = __builtin_amdgcn_readfirstlane(run_lo);
+  run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
+  tile_base = __builtin_amdgcn_readfirstlane(tile_base);
   int sb_unused;
   // part t of the request for K tile ordinal j / V tile ordinal j (nothing if the tile does not exist)
   auto request_k = [&](int j, int t) {
@@ -258,6 +278,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (GENERAL && tid < kKeyTile) {
       s_seg[buf][tid] = seg_r;
       s_pre[buf][tid] = pre_r;
+      seg_r = pre_r = 0;  // dead until the next request: not carried around the loops
     }
   };
 
@@ -434,12 +455,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT)))) {
-    int lo, hi;
+  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)))) {
+    int lo, hi;  // tile indices
     key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kKeyTile,
                          kKeyTile, lo, hi);
-    plain_lo = max(lo - j_lo, 0);
-    plain_hi = min(hi - j_lo, n);
+    plain_lo = max(lo - tile_base, run_lo);
+    plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
   }
   plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);  // wave-uniform; now the compiler knows
   plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
@@ -626,8 +647,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   const unsigned k_dst0 = RA_LDS_ADDR(&s_k[0][0]) + wave_u * 8 * (D * 2);
   const unsigned v_dst0 = RA_LDS_ADDR(&s_v[0][0]) + wave_u * 8 * (D * 2);
   auto seek_plain = [&](int ordinal) {  // the iteration with this ordinal is the next to run
-    k_run = kbase + (long long)((j_lo + ordinal + 3) * kKeyTile + 8 * wave_u) * a.k.sl;
-    v_run = vbase + (long long)((j_lo + ordinal + v_ahead) * kKeyTile + 8 * wave_u) * a.v.sl;
+    k_run = kbase + (long long)((tile_base + ordinal + 3) * kKeyTile + 8 * wave_u) * a.k.sl;
+    v_run = vbase + (long long)((tile_base + ordinal + v_ahead) * kKeyTile + 8 * wave_u) * a.v.sl;
   };
   auto sync_plain = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));  // only the previous barrier's requests are in flight
@@ -635,6 +656,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   };
   auto plain_iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
     constexpr int PAR = decltype(parity)::value;
+    constexpr int PF = GENERAL ? 2 : 3;  // the GENERAL variant has four registers less to spare
     RA_PROF_MARK(i, 1);
     if (!late_half) sync_plain();
     RA_PROF_MARK(i, 2);
@@ -704,12 +726,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       }
 #pragma unroll
       for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
+      bf16x8 q0 = qf[0];
+      if (GENERAL) q0 = s_q0[tid];
       links_of_slot(-1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int op = 0; op < NOPA; ++op) {
         if (op + PF < NOPA) fr[op + PF] = s_op_frag(kt, op + PF);
-        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
+        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? q0 : qf[op >> 1], SN[op & 1], 0, 0, 0);
         if (op == NOPA / 4) global_to_lds16_s(k_run, k_voff[0], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES);
         if (NLD == 2 && op == NOPA * 3 / 4)
           global_to_lds16_s(k_run + k_part, k_voff[NLD - 1], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES + RPI * (D * 2));
@@ -764,9 +788,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   using P3 = std::integral_constant<int, 3>;
   // iteration i is plain for plain_lo <= i < plain_end
   const int plain_end =
-      __builtin_amdgcn_readfirstlane((GENERAL || use_list || plain_hi - plain_lo < kPlainMinTiles)
+      __builtin_amdgcn_readfirstlane(plain_hi - plain_lo < kPlainMinTiles
                                          ? 0
-                                         : min(min(plain_hi - 1, n - 3), a.Lk / kKeyTile - j_lo - 3));
+                                         : min(min(plain_hi - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));
   int i = 0;
   for (; i < n && !(i >= plain_lo && i + 4 <= plain_end); i += 4) {
     iteration(P0{}, i, sa, sb);
@@ -774,13 +798,38 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
     if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
   }
-  if constexpr (!GENERAL) {  // the GENERAL variants are launched for biases that leave no plain stretch
-    if (i + 4 <= plain_end) seek_plain(i);
+  if (i + 4 <= plain_end) {
+    seek_plain(i);
+    // per-lane values that only the generic iterations use wait in LDS while the plain loop runs:
+    // it has no register to spare
+    if (GENERAL) {
+      s_stash[0][tid] = q_seg;
+      s_stash[1][tid] = q_pre;
+      s_stash[2][tid] = __float_as_int(slope2);
+      seg_r = pre_r = 0;  // already stored
+    }
     for (; i + 4 <= plain_end; i += 4) {
       plain_iteration(P0{}, i, sa, sb);
       plain_iteration(P1{}, i + 1, sb, sa);
       plain_iteration(P2{}, i + 2, sa, sb);
       plain_iteration(P3{}, i + 3, sb, sa);
+    }
+    if (GENERAL) {
+      q_seg = s_stash[0][tid];
+      q_pre = s_stash[1][tid];
+      slope2 = __int_as_float(s_stash[2][tid]);
+    }
+    // the plain iterations requested K tiles i .. i+2 without their ids: fetch them for the
+    // iterations that follow (the barrier at the top of iteration i publishes them)
+    if (GENERAL && tid < kKeyTile) {
+#pragma unroll
+      for (int t = 0; t < 3; ++t) {
+        if (i + t < n) {
+          const int kk = min(tile_at(i + t, sb_unused) * kKeyTile + tid, a.Lk - 1);
+          if (kv_seg) s_seg[(i + t) & 3][tid] = kv_seg[kk];
+          if (kv_pre) s_pre[(i + t) & 3][tid] = kv_pre[kk];
+        }
+      }
     }
   }
   for (; i < n; i += 4) {

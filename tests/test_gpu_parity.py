@@ -137,6 +137,20 @@ def test_sorted_segments_and_alibi(device):
            R.make_bias_fn(causal=True, alibi=sl))
 
 
+@pytest.mark.parametrize("causal,ring", [(False, 1), (True, 1), (True, 2)])
+def test_long_documents(device, causal, ring):
+    # documents long enough (dozens of key tiles each, boundaries off the tile grid) for the
+    # kernels to switch to their straight-line loops inside a document and back at its end
+    S = 6144
+    seg = np.zeros((1, S), np.int32)
+    seg[0, 2900:5031] = 1
+    seg[0, 5031:] = 2
+    fn = ra.segment_bias() + ra.causal_bias() if causal else ra.segment_bias()
+    _check(device, f"long-documents causal={causal}", 1, S, S, 2, 128, ring, fn,
+           R.make_bias_fn(causal=causal, use_segments=True), {"q_segment_ids": seg}, {"kv_segment_ids": seg},
+           std=0.7)
+
+
 def test_fully_masked_rows_do_not_poison_key_gradients(device):
     # queries whose segment id matches no key: o = NaN, lse = -inf like the reference
     # (ring.py:134-135); such rows must contribute nothing to dk / dv.  The expected gradients
