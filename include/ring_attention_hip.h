@@ -51,6 +51,7 @@ extern "C" {
 #define RA_BIAS_SEGMENT 4  /* q_segment_id == kv_segment_id    (ring.py:388-391)            */
 #define RA_BIAS_PREFIX 8   /* (q_prefix & kv_prefix) | kv_pos <= q_pos (ring.py:399-406)    */
 #define RA_BIAS_ALIBI 16   /* additive -slope[h] * |q_pos - kv_pos|                       */
+#define RA_BIAS_DENSE 32   /* additive fp32 block, the array a bias_fn returns (ring.py:107) */
 
 #define RA_DTYPE_BF16 0
 #define RA_DTYPE_F32 1
@@ -83,6 +84,14 @@ typedef struct ra_bias {
   int64_t q_prefix_stride_b;
   int64_t kv_prefix_stride_b;
   const float* alibi_slopes; /* [H] */
+  /* RA_BIAS_DENSE: the materialised bias of this (query shard, key/value shard) pair, exactly
+   * the `bias` argument of the reference's fwd_block / bwd_block (ring_kernel.py:127,206):
+   * fp32, element [b, h, i, j] at dense_bias[b*stride_b + h*stride_h + i*stride_q + j], added to
+   * the scaled scores (-inf masks).  stride_b / stride_h may be 0: that broadcasts the block
+   * over the batch / the heads, the reference's [b, 1, lq, lk] form.  It combines with the
+   * other terms by addition.  No gradient is produced for it (ring.py:243 returns None). */
+  const float* dense_bias;
+  int64_t dense_stride_b, dense_stride_h, dense_stride_q;
 } ra_bias;
 
 /* One ring step of the forward pass. */

@@ -47,7 +47,8 @@ int check_dims(int B, int H, int Lq, int Lk, int D) {
 }
 
 int check_bias(const ra_bias& b, int Lq, int Lk) {
-  const int known = RA_BIAS_CAUSAL | RA_BIAS_WINDOW | RA_BIAS_SEGMENT | RA_BIAS_PREFIX | RA_BIAS_ALIBI;
+  const int known = RA_BIAS_CAUSAL | RA_BIAS_WINDOW | RA_BIAS_SEGMENT | RA_BIAS_PREFIX | RA_BIAS_ALIBI |
+                    RA_BIAS_DENSE;
   if (b.flags & ~known) return fail(RA_ERR_BIAS, "unknown bias flag bits 0x%x", b.flags & ~known);
   if ((b.flags & RA_BIAS_WINDOW) && b.window <= 0)
     return fail(RA_ERR_BIAS, "window must be positive (got %d)", b.window);
@@ -61,6 +62,13 @@ int check_bias(const ra_bias& b, int Lq, int Lk) {
     return fail(RA_ERR_NULL, "prefix bias needs q_prefix and kv_prefix");
   if ((b.flags & RA_BIAS_ALIBI) && !b.alibi_slopes)
     return fail(RA_ERR_NULL, "ALiBi bias needs alibi_slopes");
+  if (b.flags & RA_BIAS_DENSE) {
+    if (!b.dense_bias) return fail(RA_ERR_NULL, "dense bias needs dense_bias");
+    if (((uintptr_t)b.dense_bias & 3) != 0) return fail(RA_ERR_ALIGN, "dense_bias is not 4-byte aligned");
+    if (b.dense_stride_q < Lk || b.dense_stride_b < 0 || b.dense_stride_h < 0)
+      return fail(RA_ERR_BIAS, "dense bias strides: stride_q must be at least Lk, stride_b / stride_h "
+                               "non-negative (0 broadcasts)");
+  }
   if (b.q_offset < 0 || b.kv_offset < 0 || b.q_offset > kMaxPos || b.kv_offset > kMaxPos)
     return fail(RA_ERR_BIAS, "token offsets must lie in [0, 2^30]");
   return RA_OK;
@@ -85,11 +93,17 @@ ra::BiasArgs to_bias(const ra_bias& b) {
   r.q_pre_sb = b.q_prefix_stride_b;
   r.kv_pre_sb = b.kv_prefix_stride_b;
   r.slopes = b.alibi_slopes;
+  r.dense = b.dense_bias;
+  r.dense_sb = b.dense_stride_b;
+  r.dense_sh = b.dense_stride_h;
+  r.dense_sq = b.dense_stride_q;
   return r;
 }
 
-bool is_general(int flags) {
-  return (flags & (RA_BIAS_SEGMENT | RA_BIAS_PREFIX | RA_BIAS_ALIBI)) != 0;
+// kernel variant: 0 = causal / window only, 1 = per-tile terms, 2 = with a dense bias block
+int kernel_mode(int flags) {
+  if (flags & RA_BIAS_DENSE) return 2;
+  return (flags & (RA_BIAS_SEGMENT | RA_BIAS_PREFIX | RA_BIAS_ALIBI)) != 0 ? 1 : 0;
 }
 
 constexpr float kLog2eHost = 1.4426950408889634f;
@@ -98,7 +112,7 @@ constexpr float kLog2eHost = 1.4426950408889634f;
 
 extern "C" {
 
-int ra_version(void) { return 1000; }
+int ra_version(void) { return 1001; }
 
 const char* ra_last_error(void) { return g_err; }
 
@@ -171,7 +185,7 @@ int ra_fwd_step(const ra_fwd_step_params* p, void* stream) {
   a.Lk = p->Lk;
   a.scale2 = p->sm_scale * kLog2eHost;
   a.bias = to_bias(p->bias);
-  hipError_t e = ra::launch_fwd_step(a, p->D, is_general(p->bias.flags), (hipStream_t)stream);
+  hipError_t e = ra::launch_fwd_step(a, p->D, kernel_mode(p->bias.flags), (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_step launch");
 }
 
@@ -232,7 +246,7 @@ int ra_bwd_step_parts(const ra_bwd_step_params* p, int32_t parts, void* stream) 
   a.scale2 = p->sm_scale * kLog2eHost;
   a.sm_scale = p->sm_scale;
   a.bias = to_bias(p->bias);
-  hipError_t e = ra::launch_bwd_step(a, p->D, is_general(p->bias.flags), parts, (hipStream_t)stream);
+  hipError_t e = ra::launch_bwd_step(a, p->D, kernel_mode(p->bias.flags), parts, (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_step launch");
 }
 

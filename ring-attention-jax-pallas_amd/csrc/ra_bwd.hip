@@ -78,8 +78,10 @@ constexpr int kQTile = 32;  // queries per LDS tile in dkdv_kernel
 // (operands visible before the barrier, so their fetch straddles it; the next tile's loads and
 // the hand-over of S(i), dP(i) to the vector ALU issue in their shadow), then the 16 MFMAs of
 // S(i+1) = Q K^T and dP(i+1) = dO V^T with the exp2 / dS arithmetic of tile i in theirs.
-template <int D, bool GENERAL>
+template <int D, int MODE>
 __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
+  constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
+  constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int NT = 256;
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
@@ -337,7 +339,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   };
   auto needs_bias = [&](int qt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (qt0 + kQTile > a.Lq);
-    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
+    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
     return nb;
   };
   constexpr int PFN = 4;  // operand fetches kept in flight ahead of the MFMA that uses them
@@ -389,15 +391,22 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
-      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
+      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE);
       if (segbit) tb.flags |= RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
+    tb.dense = nullptr;
+    tb.dense_vs = 1;
     tb.var_limit = a.Lq - (qt0 + 4 * g);
     const int rel0 = (bs.q_off + qt0 + 4 * g) - (bs.kv_off + kw + l32);
     const int* ids = (const int*)(stat_rd + ids_buf * STAT_BYTES);
-    apply_bias<false>(S, tb, rel0, k_seg, k_pre, ids + 2 * kQTile, ids + 3 * kQTile);
+    if (DENSE) {
+      tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)(qt0 + 4 * g) * bs.dense_sq +
+                 min(kw + l32, a.Lk - 1);
+      tb.dense_vs = bs.dense_sq;
+    }
+    apply_bias<false, DENSE>(S, tb, rel0, k_seg, k_pre, ids + 2 * kQTile, ids + 3 * kQTile);
   };
 
   // ---- prologue: tiles 0, 1, 2 requested, S(0) and dP(0) computed ------------------------------
@@ -415,7 +424,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   // Ordinals [plain_lo, plain_hi) of the query tiles this wave's keys see completely, unmasked
   // and in range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT)))) {
+  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT | RA_BIAS_DENSE)))) {
     int lo, hi;
     query_tile_plain_range(flags, bs.window, bs.kv_off + kw, bs.kv_off + kw + 31, bs.q_off, a.Lq / kQTile,
                            kQTile, lo, hi);
@@ -730,8 +739,10 @@ constexpr int kDqKeyTile = 32; // keys per LDS tile
 // fetch.  Iteration i, after its barrier, first runs the 8 MFMAs of dQ^T for tile i-1 (operands
 // visible before the barrier, so their fetch straddles it), then the 16 MFMAs of S^T(i+1),
 // dP^T(i+1) with the exp2 / dS arithmetic of tile i in their shadow.
-template <int D, bool GENERAL>
+template <int D, int MODE>
 __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
+  constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
+  constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
   constexpr int ROWB = D * 2;
@@ -925,7 +936,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   };
   auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (kt0 + kDqKeyTile > a.Lk);
-    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
+    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
     return nb;
   };
   constexpr int PF = 2;
@@ -963,17 +974,21 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
-      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
+      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE);
       if (segbit) tb.flags |= RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
+    tb.dense = nullptr;
+    tb.dense_vs = 1;
     const int var0 = kt0 + 4 * g;
     tb.var_limit = a.Lk - var0;
 #pragma unroll
     for (int r = 0; r < 16; ++r) S[r] *= a.scale2;
     const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
-    apply_bias<true>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
+    if (DENSE)
+      tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
+    apply_bias<true, DENSE>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
   };
 
   // ---- prologue: tiles 0, 1, 2 in flight; S^T(0), dP^T(0) computed ------------------------------
@@ -995,7 +1010,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT)))) {
+  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT | RA_BIAS_DENSE)))) {
     int lo, hi;
     key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
@@ -1265,17 +1280,20 @@ hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long lon
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, int parts, hipStream_t stream) {
+// mode: as for launch_fwd_step
+hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStream_t stream) {
   if (parts & 1) {
     const int keys_wg = 128;
     const int nkt = (a.Lk + keys_wg - 1) / keys_wg;
     dim3 grid((unsigned)(a.B * a.H * nkt)), block(256);
     if (D == 128) {
-      if (general) hipLaunchKernelGGL((dkdv_kernel<128, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dkdv_kernel<128, false>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<128, 2>), grid, block, 0, stream, a);
+      else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<128, 1>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((dkdv_kernel<128, 0>), grid, block, 0, stream, a);
     } else {
-      if (general) hipLaunchKernelGGL((dkdv_kernel<64, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dkdv_kernel<64, false>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<64, 2>), grid, block, 0, stream, a);
+      else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<64, 1>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((dkdv_kernel<64, 0>), grid, block, 0, stream, a);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -1284,11 +1302,13 @@ hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, int parts, hip
     const int nqt = (a.Lq + kDqRows - 1) / kDqRows;
     dim3 grid((unsigned)(a.B * a.H * nqt)), block(kDqThreads);
     if (D == 128) {
-      if (general) hipLaunchKernelGGL((dq_kernel<128, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dq_kernel<128, false>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dq_kernel<128, 2>), grid, block, 0, stream, a);
+      else if (mode == 1) hipLaunchKernelGGL((dq_kernel<128, 1>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((dq_kernel<128, 0>), grid, block, 0, stream, a);
     } else {
-      if (general) hipLaunchKernelGGL((dq_kernel<64, true>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dq_kernel<64, false>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dq_kernel<64, 2>), grid, block, 0, stream, a);
+      else if (mode == 1) hipLaunchKernelGGL((dq_kernel<64, 1>), grid, block, 0, stream, a);
+      else hipLaunchKernelGGL((dq_kernel<64, 0>), grid, block, 0, stream, a);
     }
   }
   return hipGetLastError();

@@ -61,6 +61,8 @@ struct BiasArgs {
   const int* kv_pre;
   long long q_pre_sb, kv_pre_sb;
   const float* slopes;
+  const float* dense;  // additive bias block [B|1, H|1, Lq, Lk], keys contiguous
+  long long dense_sb, dense_sh, dense_sq;
 };
 
 struct TensorArg {
@@ -213,9 +215,11 @@ struct TileBias {
   int window;
   float slope2;  // ALiBi slope * log2(e)
   int var_limit; // varying-side indices >= var_limit (relative to var0) are out of range
+  const float* dense;   // dense bias element of (fixed index, var0); natural-log units
+  long long dense_vs;   // its stride along the varying side (1 when the keys vary)
 };
 
-template <bool QFIXED>
+template <bool QFIXED, bool DENSE>
 RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, int fixed_pre,
                        const int* var_seg, const int* var_pre) {
 #pragma unroll
@@ -223,6 +227,12 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
     i32x4 vs = {0, 0, 0, 0}, vp = {0, 0, 0, 0};
     if (tb.flags & RA_BIAS_SEGMENT) vs = *(const i32x4*)(var_seg + 8 * bb);
     if (tb.flags & RA_BIAS_PREFIX) vp = *(const i32x4*)(var_pre + 8 * bb);
+    float dn[4] = {0.f, 0.f, 0.f, 0.f};
+    if (DENSE) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (8 * bb + c < tb.var_limit) dn[c] = QFIXED ? tb.dense[8 * bb + c] : tb.dense[(8 * bb + c) * tb.dense_vs];
+    }
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
       const int r = 4 * bb + c;
@@ -231,6 +241,7 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
       const int rel = QFIXED ? rel0 - off : rel0 + off;
       float x = t[r];
       if (tb.flags & RA_BIAS_ALIBI) x = fmaf(fabsf((float)rel), -tb.slope2, x);
+      if (DENSE) x = fmaf(dn[c], kLog2e, x);
       bool msk = off >= tb.var_limit;
       if (tb.flags & RA_BIAS_CAUSAL) msk |= rel < 0;
       if (tb.flags & RA_BIAS_WINDOW) {

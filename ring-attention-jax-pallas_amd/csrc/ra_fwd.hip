@@ -27,8 +27,10 @@ constexpr int kKeyTile = 64;    // keys per LDS tile
 constexpr int kMaxListTiles = 1024;
 constexpr int kPlainMinTiles = 16;  // shortest stretch of plain tiles that takes the straight-line loop
 
-template <int D, bool GENERAL>
+template <int D, int MODE>
 __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) {
+  constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
+  constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;  // k-steps of the QK^T contraction
   constexpr int DB = D / 32;  // 32-wide blocks of the head dim
   constexpr int TILE_BYTES = kKeyTile * D * 2;
@@ -404,7 +406,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   };
   auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (kt0 + kKeyTile > a.Lk);
-    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)) || segbit;
+    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
     return nb;
   };
   // scale + bias with the id arrays of LDS slot `ids_buf`; returns the row maximum
@@ -412,11 +414,13 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
-      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX);
+      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE);
       if (segbit) tb.flags |= RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
+    tb.dense = nullptr;
+    tb.dense_vs = 1;
     float mx = RA_NEG_INF;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
@@ -425,7 +429,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       const int var0 = kt0 + 32 * kb + 4 * g;
       tb.var_limit = a.Lk - var0;
       const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
-      apply_bias<true>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
+      if (DENSE)
+        tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
+      apply_bias<true, DENSE>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
                        &s_pre[ids_buf][32 * kb + 4 * g]);
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
@@ -455,7 +461,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX)))) {
+  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;  // tile indices
     key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kKeyTile,
                          kKeyTile, lo, hi);
@@ -923,15 +929,18 @@ __global__ void fwd_finalize_kernel(const float* o, const float* m, const float*
 // ------------------------------------------------------------------------------------------------
 namespace ra {
 
-hipError_t launch_fwd_step(const FwdArgs& a, int D, bool general, hipStream_t stream) {
+// mode: 0 = causal / window terms only, 1 = any of the per-tile terms, 2 = a dense bias block too
+hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream) {
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   dim3 grid((unsigned)(a.B * a.H * nqt)), block(kFwdThreads);
   if (D == 128) {
-    if (general) hipLaunchKernelGGL((fwd_step_kernel<128, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((fwd_step_kernel<128, false>), grid, block, 0, stream, a);
+    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<128, 2>), grid, block, 0, stream, a);
+    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<128, 1>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((fwd_step_kernel<128, 0>), grid, block, 0, stream, a);
   } else {
-    if (general) hipLaunchKernelGGL((fwd_step_kernel<64, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((fwd_step_kernel<64, false>), grid, block, 0, stream, a);
+    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<64, 2>), grid, block, 0, stream, a);
+    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<64, 1>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((fwd_step_kernel<64, 0>), grid, block, 0, stream, a);
   }
   return hipGetLastError();
 }

@@ -28,7 +28,7 @@ struct BwdArgs {
   BiasArgs bias;
 };
 
-hipError_t launch_fwd_step(const FwdArgs& a, int D, bool general, hipStream_t stream);
+hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream);
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream);
 hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, void* out, int out_f32,
                                long long sb, long long sh, long long sl, float* lse, int B, int H,
@@ -36,7 +36,7 @@ hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, v
 hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long long sh, long long sl,
                             TensorArg dout, float* delta, int B, int H, int Lq, int D,
                             hipStream_t stream);
-hipError_t launch_bwd_step(const BwdArgs& a, int D, bool general, int parts, hipStream_t stream);
+hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStream_t stream);
 hipError_t launch_mfma_rate(float* sink, int blocks, int iters, int random, hipStream_t stream);
 hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl,
                                int B, int H, int L, int D, hipStream_t stream);

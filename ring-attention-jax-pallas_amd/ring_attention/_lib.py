@@ -12,6 +12,7 @@ RA_BIAS_WINDOW = 2
 RA_BIAS_SEGMENT = 4
 RA_BIAS_PREFIX = 8
 RA_BIAS_ALIBI = 16
+RA_BIAS_DENSE = 32
 RA_DTYPE_BF16 = 0
 RA_DTYPE_F32 = 1
 
@@ -30,6 +31,8 @@ class RaBias(C.Structure):
         ("q_prefix", C.c_void_p), ("kv_prefix", C.c_void_p),
         ("q_prefix_stride_b", C.c_int64), ("kv_prefix_stride_b", C.c_int64),
         ("alibi_slopes", C.c_void_p),
+        ("dense_bias", C.c_void_p),
+        ("dense_stride_b", C.c_int64), ("dense_stride_h", C.c_int64), ("dense_stride_q", C.c_int64),
     ]
 
 

@@ -116,13 +116,16 @@ def alibi_slopes(num_heads: int) -> torch.Tensor:
 class BlockBias:
     """A BiasFn bound to ONE (query shard, key/value shard) pair: what ``bias_fn(...)``
     returns for a ring step in the reference, in un-materialised form."""
-    fn: BiasFn
+    fn: BiasFn = BiasFn()
     q_offset: int = 0
     kv_offset: int = 0
     q_segment_ids: Optional[torch.Tensor] = None   # int32 [b, lq]
     kv_segment_ids: Optional[torch.Tensor] = None  # int32 [b, lk]
     q_prefix_mask: Optional[torch.Tensor] = None   # int32 [b, lq]
     kv_prefix_mask: Optional[torch.Tensor] = None  # int32 [b, lk]
+    # materialised additive bias [b|1, h|1, lq, lk]: the array the reference's bias_fn returns and
+    # its fwd_block / bwd_block take (ring.py:107, ring_kernel.py:127); added to the other terms
+    dense: Optional[torch.Tensor] = None
 
     def to_struct(self, device) -> "_lib.RaBias":
         s = _lib.RaBias()
@@ -153,4 +156,29 @@ class BlockBias:
                 raise ValueError("alibi slopes must be moved to the compute device first")
             self._keep.append(sl)
             s.alibi_slopes = sl.data_ptr()
+        if self.dense is not None:
+            d = self.dense
+            if d.dim() != 4:
+                raise ValueError(f"a dense bias must be [b, h, lq, lk], got shape {tuple(d.shape)}")
+            if d.device != device:
+                raise ValueError(f"the dense bias must live on {device}")
+            if d.dtype != torch.float32:
+                d = d.to(torch.float32)
+            if d.stride(-1) != 1 or d.stride(2) < d.shape[3]:
+                d = d.contiguous()
+            self._keep.append(d)
+            s.flags |= _lib.RA_BIAS_DENSE
+            s.dense_bias = d.data_ptr()
+            s.dense_stride_b = 0 if d.shape[0] == 1 else d.stride(0)
+            s.dense_stride_h = 0 if d.shape[1] == 1 else d.stride(1)
+            s.dense_stride_q = d.stride(2)
         return s
+
+    def check_dense_shape(self, B: int, H: int, Lq: int, Lk: int) -> None:
+        """The broadcasting rule of the reference's block functions: [b, h | 1, lq, lk]
+        (ring_kernel.py:136-141); a batch of 1 broadcasts too."""
+        if self.dense is None:
+            return
+        sh = tuple(self.dense.shape)
+        if len(sh) != 4 or sh[0] not in (1, B) or sh[1] not in (1, H) or sh[2:] != (Lq, Lk):
+            raise ValueError(f"dense bias of shape {sh} does not broadcast to {(B, H, Lq, Lk)}")

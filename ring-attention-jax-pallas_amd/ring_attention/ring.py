@@ -12,8 +12,11 @@ Public names follow the reference (``ring.py:246`` ``ring_attention``, ``ring.py
   ``ring.py:51-55,120``.  In the backward pass the query side travels instead
   (``ring.py:195``).  The result is what ``shard_map(ring_attention)`` returns for the
   global arrays.
-* ``bias_fn`` is a declarative ``BiasFn`` (see ``bias.py``) evaluated inside the kernels;
-  ring steps and score tiles that are entirely masked are skipped.
+* ``bias_fn`` is either a declarative ``BiasFn`` (see ``bias.py``), evaluated inside the
+  kernels so that ring steps and score tiles that are entirely masked are skipped, or any
+  Python callable with the reference's contract ``bias_fn(**q_kwargs, **kv_kwargs) ->
+  [b, h | 1, lq, lk]`` (ring.py:107), whose dense block is materialised per ring step and
+  streamed by the kernels.
 * Compute is bf16 on the matrix cores with fp32 carries; other input dtypes are cast on
   entry and the result is cast back.  Head dims other than 64/128 are zero-padded.
 
@@ -25,7 +28,7 @@ from __future__ import annotations
 import ctypes as C
 import math
 from dataclasses import dataclass
-from typing import Optional, Union
+from typing import Callable, Optional, Union
 
 import torch
 
@@ -78,19 +81,26 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------------------
 # block-level API (one ring step)
 # --------------------------------------------------------------------------------------
-def _bias_struct(bias: Optional[BlockBias], device) -> _lib.RaBias:
+def _bias_struct(bias, device, shape=None) -> _lib.RaBias:
+    """``bias`` is None, a ``BlockBias`` or a dense additive array ``[b, h | 1, lq, lk]`` - the
+    form the reference's block functions take (ring_kernel.py:127,206)."""
     if bias is None:
         return _lib.RaBias()
+    if isinstance(bias, torch.Tensor):
+        bias = BlockBias(dense=bias)
+    if shape is not None:
+        bias.check_dense_shape(*shape)
     return bias.to_struct(device)
 
 
-def fwd_block(q, k, v, bias: Optional[BlockBias], o, m, l, sm_scale: float):
+def fwd_block(q, k, v, bias: Union[BlockBias, torch.Tensor, None], o, m, l, sm_scale: float):
     """One ring step of the forward pass, in place on the fp32 carry.
 
     Same contract as the reference's ``fwd_block`` (ring_kernel.py:123-199): ``q`` is
     ``[b, h, lq, d]``, ``k``/``v`` are ``[b, h, lk, d]`` (bf16, any batch/head/length strides),
     ``o`` ``[b, h, lq, d]`` is the unnormalised output and ``m``/``l`` ``[b, h, lq]`` the
-    running max / sum (fp32, contiguous).  ``bias`` describes the block's additive bias.
+    running max / sum (fp32, contiguous).  ``bias`` is the block's additive bias: a dense
+    ``[b, h | 1, lq, lk]`` array as in the reference, or a ``BlockBias`` description.
     Returns ``(o, m, l)`` (the same tensors, updated)."""
     _require_gpu(q)
     lib = _lib.load()
@@ -103,7 +113,7 @@ def fwd_block(q, k, v, bias: Optional[BlockBias], o, m, l, sm_scale: float):
         if t_.dtype != torch.float32 or not t_.is_contiguous():
             raise ValueError("o, m, l carries must be contiguous float32 tensors")
     p.o, p.m, p.l = o.data_ptr(), m.data_ptr(), l.data_ptr()
-    p.bias = _bias_struct(bias, q.device)
+    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
     _lib.check("ra_fwd_step", lib.ra_fwd_step(C.byref(p), _stream()))
     return o, m, l
 
@@ -161,11 +171,11 @@ def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, parts=3):
     p.q, p.k, p.v, p.dout = _view_bhld(q), _view_bhld(k), _view_bhld(v), _view_bhld(do)
     p.lse, p.delta = lse.data_ptr(), delta.data_ptr()
     p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
-    p.bias = _bias_struct(bias, q.device)
+    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
     _lib.check("ra_bwd_step", lib.ra_bwd_step_parts(C.byref(p), parts, _stream()))
 
 
-def bwd_block(q, k, v, bias: Optional[BlockBias], o, L, do, sm_scale: float):
+def bwd_block(q, k, v, bias: Union[BlockBias, torch.Tensor, None], o, L, do, sm_scale: float):
     """Gradients of one (query block, key/value block) pair, as the reference's
     ``bwd_block`` (ring_kernel.py:202-297): all tensors ``[b, h, l, d]``, ``o`` the normalised
     forward output, ``L`` the logsumexp ``[b, h, lq]``.  Returns fp32 ``(dq, dk, dv)``."""
@@ -200,9 +210,25 @@ class _RingPlan:
             raise ValueError(f"sequence lengths ({Sq}, {Sk}) must be divisible by the ring size {n}")
         self.Lq, self.Lk = Sq // n, Sk // n
         self.fn = fn
+        self.callable = None
         dev = q.device
         q_kwargs = dict(q_kwargs or {})
         kv_kwargs = dict(kv_kwargs or {})
+        self.q_off = [r * self.Lq for r in range(n)]
+        self.kv_off = [r * self.Lk for r in range(n)]
+        if fn is not None and not isinstance(fn, BiasFn):
+            # The reference's general form (ring.py:107,186): any callable of per-token arrays.
+            # Every kwarg is an array whose axis 1 is the sequence; its shards travel with the
+            # query / key-value shards exactly as bias_q_kwargs / bias_kv_kwargs do there.
+            for name, t in list(q_kwargs.items()) + list(kv_kwargs.items()):
+                S = Sq if name in q_kwargs else Sk
+                if not isinstance(t, torch.Tensor) or t.dim() < 2 or t.shape[1] != S:
+                    raise ValueError(f"bias kwarg {name!r} must be a tensor [b, {S}, ...]")
+            self.callable = fn
+            self.fn = None
+            self.q_kw = {a: t.to(dev) for a, t in q_kwargs.items()}
+            self.kv_kw = {a: t.to(dev) for a, t in kv_kwargs.items()}
+            return
         known_q = {"q_segment_ids", "q_positions", "q_prefix_mask"}
         known_kv = {"kv_segment_ids", "kv_positions", "kv_prefix_mask"}
         for name in list(q_kwargs) + list(kv_kwargs):
@@ -220,8 +246,6 @@ class _RingPlan:
             return t.to(device=dev, dtype=torch.int32).contiguous()
 
         self.q_seg = self.kv_seg = self.q_pre = self.kv_pre = None
-        self.q_off = [r * self.Lq for r in range(n)]
-        self.kv_off = [r * self.Lk for r in range(n)]
         if fn is not None:
             fn.validate()
             if fn.segments:
@@ -261,10 +285,16 @@ class _RingPlan:
 
     def block_bias(self, qs: int, ks: int) -> Optional[BlockBias]:
         """Bias of (query shard qs, key/value shard ks)."""
-        if self.fn is None:
-            return None
         sl_q = slice(qs * self.Lq, (qs + 1) * self.Lq)
         sl_k = slice(ks * self.Lk, (ks + 1) * self.Lk)
+        if self.callable is not None:
+            dense = self.callable(**{a: t[:, sl_q] for a, t in self.q_kw.items()},
+                                  **{a: t[:, sl_k] for a, t in self.kv_kw.items()})
+            if not isinstance(dense, torch.Tensor):
+                raise TypeError("a callable bias_fn must return a torch.Tensor [b, h | 1, lq, lk]")
+            return BlockBias(dense=dense)
+        if self.fn is None:
+            return None
         return BlockBias(
             self.fn, self.q_off[qs], self.kv_off[ks],
             None if self.q_seg is None else self.q_seg[:, sl_q],
@@ -371,16 +401,16 @@ class _RingAttentionFn(torch.autograd.Function):
         return dq, dk, dv, None, None, None
 
 
-def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Optional[BiasFn] = None, bias_q_kwargs=None,
+def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = None, bias_q_kwargs=None,
                             bias_kv_kwargs=None, sm_scale: Optional[float] = None,
                             block_impl: str = "hip", out_dtype=None):
     """``ring_attention`` that also returns the logsumexp ``[b, h, S]`` (the ``L`` residual of
     ring.py:135)."""
     if block_impl not in _IMPLS:
         raise ValueError(block_impl)
-    if bias_fn is not None and not isinstance(bias_fn, BiasFn):
-        raise TypeError("bias_fn must be a ring_attention.BiasFn: arbitrary Python callables "
-                        "cannot be evaluated inside the kernels")
+    if bias_fn is not None and not isinstance(bias_fn, BiasFn) and not callable(bias_fn):
+        raise TypeError("bias_fn must be a ring_attention.BiasFn or a callable returning the dense "
+                        "[b, h | 1, lq, lk] bias of a block")
     _require_gpu(q)
     _lib.load()
     n = _axis_size(axis_name)
@@ -411,16 +441,20 @@ def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Optional[BiasFn] = None
     return out, lse_full
 
 
-def ring_attention(q, k, v, axis_name, bias_fn: Optional[BiasFn] = None, bias_q_kwargs=None,
+def ring_attention(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = None, bias_q_kwargs=None,
                    bias_kv_kwargs=None, sm_scale: Optional[float] = None, block_impl: str = "hip"):
     """Ring attention - general (reference ``ring_attention``, ring.py:246-325).
 
     Args:
         q, k, v: ``[b, S, h, d]`` global arrays on the GPU (see the module docstring).
         axis_name: ``RingAxis`` / int ring size: how many shards the sequence is cut into.
-        bias_fn: optional ``BiasFn`` describing the block-wise attention bias.
-        bias_q_kwargs / bias_kv_kwargs: query- / key-aligned ``[b, S]`` arrays the bias needs
-            (``q_segment_ids``, ``q_positions``, ``q_prefix_mask`` and their ``kv_`` twins).
+        bias_fn: optional block-wise attention bias: a ``BiasFn`` description (evaluated inside the
+            kernels, masked tiles skipped) or, as in the reference, any callable
+            ``bias_fn(**q_kwargs, **kv_kwargs)`` returning the additive ``[b, h | 1, lq, lk]`` block
+            of one (query shard, key/value shard) pair; no gradient flows into it (ring.py:243).
+        bias_q_kwargs / bias_kv_kwargs: query- / key-aligned ``[b, S, ...]`` arrays the bias needs;
+            for a ``BiasFn``: ``q_segment_ids``, ``q_positions``, ``q_prefix_mask`` and their
+            ``kv_`` twins.
         sm_scale: softmax scale, 1/sqrt(d) if unspecified.
         block_impl: ``"hip"`` (``"pallas"`` is accepted as an alias); anything else raises
             ``ValueError`` as the reference does (ring.py:312).

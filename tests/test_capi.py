@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol(lib):
 def test_struct_layout_matches_header():
     # sizes implied by the header with natural alignment on x86-64
     assert C.sizeof(_lib.RaTensor) == 32
-    assert C.sizeof(_lib.RaBias) == 8 + 16 + 16 + 16 + 16 + 16 + 8
+    assert C.sizeof(_lib.RaBias) == 8 + 16 + 16 + 16 + 16 + 16 + 8 + 8 + 24
     assert C.sizeof(_lib.RaFwdStepParams) == 24 + 3 * 32 + 24 + C.sizeof(_lib.RaBias)
     assert C.sizeof(_lib.RaBwdStepParams) == 24 + 4 * 32 + 40 + C.sizeof(_lib.RaBias)
 
@@ -78,6 +78,11 @@ def test_check_accepts_good_params(lib):
     (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL | _lib.RA_BIAS_PREFIX), -5),
     (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_SEGMENT), -1),           # no id arrays
     (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_ALIBI), -1),             # no slopes
+    (lambda p: setattr(p.bias, "flags", _lib.RA_BIAS_DENSE), -1),             # no dense block
+    (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_DENSE), setattr(p.bias, "dense_bias", 0x3000),
+                setattr(p.bias, "dense_stride_q", 63)), -5),                  # rows overlap
+    (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_DENSE), setattr(p.bias, "dense_bias", 0x3002),
+                setattr(p.bias, "dense_stride_q", 64)), -4),
     (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL), setattr(p.bias, "q_offset", -5)), -5),
 ])
 def test_fwd_step_rejects_bad_params_without_a_gpu(lib, mutate, code):

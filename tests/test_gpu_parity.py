@@ -264,6 +264,109 @@ def test_block_api_matches_reference_contract(device):
         assert mx <= GRAD_TOL and fro <= GRAD_TOL
 
 
+# ---- arbitrary bias_fn callables: the dense additive block of ring.py:107 ---------------------------
+def _callable_check(device, name, B, Sq, Sk, H, D, n, torch_fn, numpy_fn, qkw, kvkw, seed=0):
+    """ring_attention with a Python callable as bias_fn against the dense closed form with the
+    same function evaluated by numpy on the whole sequence."""
+    print(f"[parity] {name}: B={B} Sq={Sq} Sk={Sk} H={H} D={D} ring={n}", flush=True)
+    q, k, v, do = R.make_inputs(seed, B, Sq, Sk, H, D)
+    out, lse, g = _run_hip(device, q, k, v, do, n, torch_fn, qkw, kvkw)
+    bias = numpy_fn(**qkw, **kvkw)
+    want, want_lse = R.mha_dense(q, k, v, bias)
+    np.testing.assert_array_equal(np.isnan(out), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.abs(out - want)[ok].max() <= OUT_TOL
+    okl = np.isfinite(want_lse)
+    assert np.abs(lse[okl] - want_lse[okl]).max() <= LSE_TOL
+    if ok.all():
+        for got, ref, nm in zip(g, R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
+            mx, fro = _rel(got, ref)
+            assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+
+
+@pytest.mark.parametrize("seed,q_len,kv_len,h,d", [(1, 128, 64, 4, 64), (2, 64, 512, 4, 16), (3, 2048, 2048, 4, 128)])
+def test_callable_segment_bias_fn(device, seed, q_len, kv_len, h, d):
+    # the bias_fn of the reference's own test (ring_test.py:226-246): a callable that builds the
+    # [b, 1, lq, lk] mask block from the two id arrays
+    rng = np.random.default_rng(seed)
+    qs = rng.integers(0, 5, (2, q_len)).astype(np.int32)
+    ks = rng.integers(0, 5, (2, kv_len)).astype(np.int32)
+
+    def torch_fn(q_segment_ids, kv_segment_ids):
+        same = q_segment_ids[:, None, :, None] == kv_segment_ids[:, None, None, :]
+        return torch.where(same, 0.0, -torch.inf)
+
+    def numpy_fn(q_segment_ids, kv_segment_ids):
+        same = q_segment_ids[:, None, :, None] == kv_segment_ids[:, None, None, :]
+        return np.where(same, 0.0, -np.inf)
+
+    _callable_check(device, "callable-segments", 2, q_len, kv_len, h, d, 8, torch_fn, numpy_fn,
+                    {"q_segment_ids": qs}, {"kv_segment_ids": ks}, seed=seed)
+
+
+def test_callable_per_head_finite_bias_fn(device):
+    # a finite per-head bias of arbitrary per-token features (not expressible by the built-in
+    # terms), ragged shard length, plus a causal mask folded into the same callable
+    B, S, H, D, n = 2, 3 * 200, 3, 64, 3
+    rng = np.random.default_rng(7)
+    qf = rng.standard_normal((B, S, H)).astype(np.float32)
+    kf = rng.standard_normal((B, S, H)).astype(np.float32)
+    pos = np.broadcast_to(np.arange(S, dtype=np.int32), (B, S)).copy()
+
+    def torch_fn(q_feat, q_pos, kv_feat, kv_pos):
+        bias = torch.einsum("bqh,bkh->bhqk", q_feat, kv_feat)
+        return bias.masked_fill(kv_pos[:, None, None, :] > q_pos[:, None, :, None], -torch.inf)
+
+    def numpy_fn(q_feat, q_pos, kv_feat, kv_pos):
+        bias = np.einsum("bqh,bkh->bhqk", q_feat.astype(np.float64), kv_feat.astype(np.float64))
+        return np.where(kv_pos[:, None, None, :] > q_pos[:, None, :, None], -np.inf, bias)
+
+    _callable_check(device, "callable-per-head", B, S, S, H, D, n, torch_fn, numpy_fn,
+                    {"q_feat": qf, "q_pos": pos}, {"kv_feat": kf, "kv_pos": pos})
+
+
+def test_block_api_dense_bias(device):
+    """fwd_block / bwd_block with the dense [b, 1, lq, lk] bias array the reference's block
+    functions take (ring_kernel.py:127,136-141), broadcast over the heads, rows fully masked."""
+    B, H, Lq, Lk, D = 2, 3, 200, 333, 128
+    q, k, v, do = R.make_inputs(11, B, Lq, Lk, H, D)
+    rng = np.random.default_rng(11)
+    bias = rng.standard_normal((B, 1, Lq, Lk)).astype(np.float32)
+    bias[rng.random((B, 1, Lq, Lk)) < 0.3] = -np.inf
+    bias[:, :, 17, :] = -np.inf  # a query without any key: carry untouched, l stays 0
+    hq, hk, hv, hdo = (np.ascontiguousarray(np.transpose(x, (0, 2, 1, 3))) for x in (q, k, v, do))
+    tq, tk, tv, tdo = (_dev(x, device, torch.bfloat16) for x in (hq, hk, hv, hdo))
+    tb = _dev(bias, device)
+    o, m, l = rr.init_carry(B, H, Lq, D, device)
+    scale = 1 / math.sqrt(D)
+    o, m, l = ra.fwd_block(tq, tk, tv, tb, o, m, l, scale)
+    f64 = lambda x: x.astype(np.float64)
+    wo, wm, wl = R.fwd_block(f64(hq), f64(hk), f64(hv), f64(bias), np.zeros((B, H, Lq, D)),
+                             np.full((B, H, Lq), -np.inf), np.zeros((B, H, Lq)), scale)
+    assert torch.all(l[:, :, 17] == 0) and torch.all(torch.isneginf(m[:, :, 17]))
+    live = np.ones(Lq, bool)
+    live[17] = False
+    assert np.abs(m.cpu().numpy()[:, :, live] - wm[:, :, live]).max() <= 1e-4
+    np.testing.assert_allclose(l.cpu().numpy()[:, :, live], wl[:, :, live], rtol=5e-3)
+    got_out = (o / l[..., None]).cpu().numpy()[:, :, live]
+    assert np.abs(got_out - wo[:, :, live] / wl[:, :, live, None]).max() <= OUT_TOL
+    # backward on the live rows (the reference's block would divide by zero on row 17)
+    out = torch.where(l[..., None] > 0, o / l[..., None], torch.zeros_like(o))
+    L = m + torch.log(l)
+    dq, dk, dv = ra.bwd_block(tq, tk, tv, tb, out, L, tdo, scale)
+    wout = np.where(wl[..., None] > 0, wo / np.where(wl > 0, wl, 1)[..., None], 0.0)
+    wL = np.where(wl > 0, wm + np.log(np.where(wl > 0, wl, 1)), -np.inf)
+    sel = np.ix_(range(B), range(H), np.nonzero(live)[0])
+    wdq, wdk, wdv = R.bwd_block(f64(hq)[sel], f64(hk), f64(hv), f64(bias)[:, :, live], wout[sel], wL[sel],
+                                f64(hdo)[sel], scale)
+    assert torch.all(dq[:, :, 17] == 0)
+    for got, ref in ((dq.cpu().numpy()[sel], wdq), (dk.cpu().numpy(), wdk), (dv.cpu().numpy(), wdv)):
+        mx, fro = _rel(got, ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL
+    with pytest.raises(ValueError):
+        ra.fwd_block(tq, tk, tv, tb[:, :, :, :-1], o, m, l, scale)
+
+
 def test_delta_kernel(device):
     B, H, L, D = 2, 3, 100, 64
     rng = np.random.default_rng(0)

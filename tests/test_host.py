@@ -38,7 +38,7 @@ def test_block_impl_and_bias_type_errors():
     with pytest.raises(ValueError):
         ra.ring_attention(q, q, q, 2, block_impl="jax")  # ring.py:312 raises ValueError too
     with pytest.raises(TypeError):
-        ra.ring_attention(q, q, q, 2, bias_fn=lambda **kw: None)
+        ra.ring_attention(q, q, q, 2, bias_fn="causal")  # neither a BiasFn nor a callable
     with pytest.raises(TypeError):
         rr._axis_size("sp")
     assert rr._axis_size(ra.RingAxis("sp", 8)) == 8 and rr._axis_size(("sp", 4)) == 4
@@ -83,6 +83,33 @@ def test_ring_plan_shards_and_offsets():
         rr._RingPlan(q, k, 4, ra.causal_bias(), {"bogus": seg_q}, {})
     with pytest.raises(ValueError):
         rr._RingPlan(q, k, 4, None, {"q_segment_ids": seg_q}, {})
+
+
+def test_ring_plan_with_a_callable_bias_fn():
+    # the reference's general form: the callable sees the shards of its kwargs (ring.py:107,186)
+    q = torch.zeros(2, 64, 2, 64, dtype=torch.bfloat16)
+    k = torch.zeros(2, 32, 2, 64, dtype=torch.bfloat16)
+    feat_q = torch.arange(2 * 64 * 3, dtype=torch.float32).reshape(2, 64, 3)
+    ids_k = torch.arange(32)[None].repeat(2, 1)
+    seen = {}
+
+    def fn(q_feat, kv_ids):
+        seen["q"], seen["k"] = q_feat, kv_ids
+        return torch.zeros(2, 1, q_feat.shape[1], kv_ids.shape[1])
+
+    plan = rr._RingPlan(q, k, 4, fn, {"q_feat": feat_q}, {"kv_ids": ids_k})
+    bb = plan.block_bias(2, 3)
+    assert torch.equal(seen["q"], feat_q[:, 32:48]) and torch.equal(seen["k"], ids_k[:, 24:32])
+    assert bb.dense.shape == (2, 1, 16, 8) and bb.fn.flags == 0
+    bb.check_dense_shape(2, 2, 16, 8)
+    with pytest.raises(ValueError):
+        bb.check_dense_shape(2, 2, 16, 9)
+    s = bb.to_struct(torch.device("cpu"))
+    assert s.flags == 32 and s.dense_stride_h == 0 and s.dense_stride_q == 8 and s.dense_stride_b == 128
+    with pytest.raises(ValueError):
+        rr._RingPlan(q, k, 4, fn, {"q_feat": feat_q[:, :10]}, {"kv_ids": ids_k})
+    with pytest.raises(TypeError):
+        rr._RingPlan(q, k, 4, lambda **kw: None, {}, {}).block_bias(0, 0)
 
 
 def test_shard_view_is_zero_copy():
