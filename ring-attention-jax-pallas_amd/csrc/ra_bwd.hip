@@ -163,6 +163,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   query_tile_range(flags, bs.window, bs.kv_off + k0, bs.kv_off + k_hi, bs.q_off, ntiles, kQTile, i_lo, i_hi);
   int n_act = i_hi - i_lo;
   bool use_list = false;
+  // ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` that need no segment test
+  int run_lo = 0, run_hi = n_act, tile_base = i_lo;
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     use_list = true;
     int smin = 0x7fffffff, smax = (int)0x80000000;
@@ -184,13 +186,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       kmax = max(kmax, s_red[4 + w]);
     }
     for (int i = i_lo + tid; i < i_hi; i += NT) {
-      int qmin = 0x7fffffff, qmax = (int)0x80000000;
-      const int qend = min((i + 1) * kQTile, a.Lq);
-      for (int qq = i * kQTile; qq < qend; ++qq) {
-        int sid = q_seg[qq];
-        qmin = min(qmin, sid);
-        qmax = max(qmax, sid);
-      }
+      int qmin, qmax;
+      tile_id_range<kQTile>(q_seg, i, a.Lq, qmin, qmax);
       const bool act = !(qmax < kmin || qmin > kmax);
       const bool uniform = (kmin == kmax) && (qmin == qmax) && (kmin == qmin);
       s_flag[i - i_lo] = act ? (uniform ? 1 : 3) : 0;
@@ -205,12 +202,25 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
         if (f) s_list[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)((i_lo + i) | ((f & 2) << 14));
         cnt += __popcll(mask);
       }
-      if (lane == 0) s_red[8] = cnt;
+      int u_lo, u_hi, u_base;
+      uniform_run(s_list, cnt, lane, u_lo, u_hi, u_base);
+      if (lane == 0) {
+        s_red[8] = cnt;
+        s_red[9] = u_lo;
+        s_red[10] = u_hi;
+        s_red[11] = u_base;
+      }
     }
     __syncthreads();
     n_act = s_red[8];
+    run_lo = s_red[9];
+    run_hi = s_red[10];
+    tile_base = s_red[11];
   }
-  const int n = n_act;
+  const int n = __builtin_amdgcn_readfirstlane(n_act);
+  run_lo = __builtin_amdgcn_readfirstlane(run_lo);
+  run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
+  tile_base = __builtin_amdgcn_readfirstlane(tile_base);
 
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
@@ -424,12 +434,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   // Ordinals [plain_lo, plain_hi) of the query tiles this wave's keys see completely, unmasked
   // and in range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT | RA_BIAS_DENSE)))) {
+  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
     query_tile_plain_range(flags, bs.window, bs.kv_off + kw, bs.kv_off + kw + 31, bs.q_off, a.Lq / kQTile,
                            kQTile, lo, hi);
-    plain_lo = max(lo - i_lo, 0);
-    plain_hi = min(hi - i_lo, n);
+    plain_lo = max(lo - tile_base, run_lo);
+    plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
   }
   plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);
   plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
@@ -668,7 +678,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
   // iteration i is plain for plain_lo < i < plain_end (tile i+3 must exist and be complete)
-  const int plain_end = GENERAL ? -1 : min(min(plain_hi - 1, n - 3), a.Lq / kQTile - i_lo - 3);
+  const int plain_end = __builtin_amdgcn_readfirstlane(
+      DENSE ? -1 : min(min(plain_hi - 1, run_hi - 3), a.Lq / kQTile - tile_base - 3));
   int i = 0;
   for (; i < n && !(i > plain_lo && i + NB <= plain_end); i += NB) {
     iteration(P0{}, i);
@@ -678,8 +689,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (i + 4 < n) iteration(P4{}, i + 4);
     if (i + 5 < n) iteration(P5{}, i + 5);
   }
-  if constexpr (!GENERAL) {  // the GENERAL variants are launched for biases that leave no plain stretch
-    if (i + NB <= plain_end) seek_plain(i_lo + i + 3);
+  if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+    if (i + NB <= plain_end) seek_plain(tile_base + i + 3);
     for (; i + NB <= plain_end; i += NB) {
       plain_iteration(P0{}, i);
       plain_iteration(P1{}, i + 1);
@@ -710,17 +721,37 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 
   RA_PROF_DUMP;
   // ---- accumulate into the fp32 gradients owned by this key slab ------------------------------
+  // All loads of an array are issued before the first value is needed: a load - add - store chain
+  // per element would cost one memory round trip each, a hundred in a row with nothing to hide them.
+  {
+    float* const dkp = a.dk + (((long long)b * a.H + h) * a.Lk + kw + 4 * g) * D + l32;
+    float* const dvp = a.dv + (((long long)b * a.H + h) * a.Lk + kw + 4 * g) * D + l32;
+    const int key0 = kw + 4 * g;
+    auto add_to = [&](float* p, const f32x16 (&acc)[DB], float mul) {
+      float old[DB][16];
+      if (kw + 32 <= a.Lk) {  // the whole wave is in range (wave-uniform): straight-line code
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const int key = kw + 8 * (r / 4) + 4 * g + (r % 4);
-    if (key < a.Lk) {
-      const long long off = (((long long)b * a.H + h) * a.Lk + key) * D + l32;
+        for (int r = 0; r < 16; ++r)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        a.dk[off + 32 * db] += dk[db][r] * a.sm_scale;
-        a.dv[off + 32 * db] += dv[db][r];
+          for (int db = 0; db < DB; ++db) old[db][r] = p[(8 * (r / 4) + (r % 4)) * D + 32 * db];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+            p[(8 * (r / 4) + (r % 4)) * D + 32 * db] = fmaf(acc[db][r], mul, old[db][r]);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kr = 8 * (r / 4) + (r % 4);
+          if (key0 + kr < a.Lk) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) p[kr * D + 32 * db] += acc[db][r] * mul;
+          }
+        }
       }
-    }
+    };
+    add_to(dkp, dk, a.sm_scale);
+    add_to(dvp, dv, 1.0f);
   }
 }
 
@@ -756,6 +787,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[20];
+  // The GENERAL variants are a few registers short in their straight-line loop: the first operand
+  // fragments of Q and dO and the per-lane load offsets wait here and are fetched once per
+  // iteration instead (a spill to scratch memory would make every iteration wait for all loads).
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q0[GENERAL ? kDqThreads : 1];
+  __shared__ __attribute__((aligned(16))) bf16x8 s_do0[GENERAL ? kDqThreads : 1];
+  __shared__ __attribute__((aligned(8))) unsigned s_voff[GENERAL ? kDqThreads : 1][2];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -782,6 +819,10 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     for (int s = 0; s < KS; ++s) {
       qf[s] = *(const bf16x8*)(qp + 16 * s);
       dof[s] = *(const bf16x8*)(dp + 16 * s);
+    }
+    if (GENERAL) {
+      s_q0[tid] = qf[0];
+      s_do0[tid] = dof[0];
     }
   }
   const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
@@ -812,6 +853,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
+  // ordinals [run_lo, run_hi) are tiles that need no segment test
+  int run_lo = 0, run_hi = n_act;
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     use_list = true;
     int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
@@ -829,13 +872,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       qmax = max(qmax, s_red[8 + w]);
     }
     for (int j = j_lo + tid; j < j_hi; j += kDqThreads) {
-      int kmin = 0x7fffffff, kmax = (int)0x80000000;
-      const int kend = min((j + 1) * kDqKeyTile, a.Lk);
-      for (int kk = j * kDqKeyTile; kk < kend; ++kk) {
-        int sid = kv_seg[kk];
-        kmin = min(kmin, sid);
-        kmax = max(kmax, sid);
-      }
+      int kmin, kmax;
+      tile_id_range<kDqKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
       const bool act = !(kmax < qmin || kmin > qmax);
       const bool uniform = (kmin == kmax) && (qmin == qmax) && (kmin == qmin);
       s_flag[j - j_lo] = act ? (uniform ? 1 : 3) : 0;
@@ -850,12 +888,22 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
         if (f) s_list[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)((j_lo + i) | ((f & 2) << 14));
         cnt += __popcll(mask);
       }
-      if (lane == 0) s_red[16] = cnt;
+      int u_lo, u_hi, u_base;
+      uniform_run(s_list, cnt, lane, u_lo, u_hi, u_base);
+      if (lane == 0) {
+        s_red[16] = cnt;
+        s_red[17] = u_lo;
+        s_red[18] = u_hi;
+      }
     }
     __syncthreads();
     n_act = s_red[16];
+    run_lo = s_red[17];
+    run_hi = s_red[18];
   }
-  const int n = n_act;
+  const int n = __builtin_amdgcn_readfirstlane(n_act);
+  run_lo = __builtin_amdgcn_readfirstlane(run_lo);
+  run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
 
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
@@ -878,22 +926,31 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   const int ld_chunk = ((tile_off<D>(ld_row, lane % CPR) - ld_row * ROWB) >> 4) * 8;
   const unsigned k_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.k.sl + ld_chunk) * 2);
   const unsigned v_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.v.sl + ld_chunk) * 2);
+  if (GENERAL) {
+    s_voff[tid][0] = k_voff;
+    s_voff[tid][1] = v_voff;
+  }
   int seg_r = 0, pre_r = 0;
-  auto issue_tile = [&](int j, int buf) {
+  auto issue_tile = [&](int j, int buf, bool with_ids = true) {
     const int k0 = j * kDqKeyTile;
+    unsigned kvo = k_voff, vvo = v_voff;
+    if (GENERAL && !with_ids) {  // called from the straight-line loop
+      kvo = s_voff[tid][0];
+      vvo = s_voff[tid][1];
+    }
     const unsigned k_dst = RA_LDS_ADDR(&s_k[0][0]) + buf * TILE_BYTES + wave_u * RPW * ROWB;
     const unsigned v_dst = RA_LDS_ADDR(&s_v[0][0]) + buf * TILE_BYTES + wave_u * RPW * ROWB;
     if (ld_lane_on) {
       if (k0 + kDqKeyTile <= a.Lk) {
-        global_to_lds16_s(kbase + (long long)(k0 + RPW * wave_u) * a.k.sl, k_voff, k_dst);
-        global_to_lds16_s(vbase + (long long)(k0 + RPW * wave_u) * a.v.sl, v_voff, v_dst);
+        global_to_lds16_s(kbase + (long long)(k0 + RPW * wave_u) * a.k.sl, kvo, k_dst);
+        global_to_lds16_s(vbase + (long long)(k0 + RPW * wave_u) * a.v.sl, vvo, v_dst);
       } else {  // last, partial tile: rows past the end repeat the last row (masked later)
         const int gr = min(k0 + ld_row, a.Lk - 1);
         global_to_lds16(kbase + (long long)gr * a.k.sl + ld_chunk, k_dst);
         global_to_lds16(vbase + (long long)gr * a.v.sl + ld_chunk, v_dst);
       }
     }
-    if (GENERAL && tid < kDqKeyTile) {
+    if (GENERAL && with_ids && tid < kDqKeyTile) {
       int kk = min(k0 + tid, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
@@ -1010,12 +1067,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !use_list && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_SEGMENT | RA_BIAS_DENSE)))) {
+  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
     key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
-    plain_lo = max(lo - j_lo, 0);
-    plain_hi = min(hi - j_lo, n);
+    // ordinal of tile t inside the run: t - (first tile of the run) + run_lo
+    int sbu;
+    const int run_tile0 = (run_hi > run_lo) ? tile_at(run_lo, sbu) - run_lo : j_lo;
+    plain_lo = max(lo - run_tile0, run_lo);
+    plain_hi = max(min(hi - run_tile0, run_hi), plain_lo);
   }
 
   plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);
@@ -1110,8 +1170,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     for (int op = 0; op < PF; ++op) frb[op] = tr_frag(kp, op / DB, op % DB);
     if (!late_half) {
       // all loads but the two of tile i+2 have landed: this wave's share of tile i+1 is in LDS
-      if (GENERAL) __builtin_amdgcn_s_waitcnt(0x0f70);
-      else __builtin_amdgcn_s_waitcnt(0x0f72);
+      __builtin_amdgcn_s_waitcnt(0x0f72);
       __syncthreads();
     }
     RA_PROFQ_MARK(i, 2);
@@ -1132,7 +1191,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       acc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frb[op], dsf[op / DB], acc[op % DB], 0, 0, 0);
       if (op == 0) {  // next loads: their issue hides behind the MFMAs
         int sbu;
-        issue_tile(tile_at(i + 3, sbu), PH3);
+        issue_tile(tile_at(i + 3, sbu), PH3, false);  // plain tiles: nobody reads their ids
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1140,13 +1199,17 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       // this half of the workgroup meets the barrier here, so that on every SIMD one wave runs
       // its dQ^T block while the other runs its S^T / dP^T block.  Tiles i+2 and i+3 may still
       // be in flight (two loads each).
-      if (GENERAL) __builtin_amdgcn_s_waitcnt(0x0f70);
-      else __builtin_amdgcn_s_waitcnt(0x0f74);
+      __builtin_amdgcn_s_waitcnt(0x0f74);
       __syncthreads();
 #pragma unroll
       for (int op = 0; op < PF; ++op) fra[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
     }
     RA_PROFQ_MARK(i, 3);
+    bf16x8 q0 = qf[0], do0 = dof[0];
+    if (GENERAL) {
+      q0 = s_q0[tid];
+      do0 = s_do0[tid];
+    }
     float ds_prev = 0.f;
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
@@ -1155,8 +1218,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
         f32x16 z;
 #pragma unroll
         for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], dof[op >> 1], z, 0, 0, 0);
-        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], qf[op >> 1], z, 0, 0, 0);
+        if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], do0, z, 0, 0, 0);
+        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], q0, z, 0, 0, 0);
       } else {
         if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], dof[op >> 1], PN, 0, 0, 0);
         else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], qf[op >> 1], SN, 0, 0, 0);
@@ -1190,7 +1253,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   using P3 = std::integral_constant<int, 3>;
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
-  const int plain_end = GENERAL ? -1 : min(plain_hi - 1, n - 3);  // iteration i is plain for plain_lo < i < plain_end
+  // iteration i is plain for plain_lo < i < plain_end
+  const int plain_end = __builtin_amdgcn_readfirstlane(DENSE ? -1 : min(plain_hi - 1, min(run_hi, n) - 3));
   int i = 0;
   for (; i < n && !(i > plain_lo && i + 6 <= plain_end); i += 6) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
@@ -1200,7 +1264,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  if constexpr (!GENERAL) {  // the GENERAL variants are launched for biases that leave no plain stretch
+  if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+    const bool stretch = i + 6 <= plain_end;
+    if (GENERAL && stretch) seg_r = pre_r = 0;  // stored already; not carried through the stretch
     for (; i + 6 <= plain_end; i += 6) {
       plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
       plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
@@ -1208,6 +1274,22 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
       plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
       plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+    }
+    if (GENERAL && stretch && tid < kDqKeyTile) {
+      // the stretch moved no ids: those of the two tiles in flight are fetched now (i is a
+      // multiple of 6 here: tile i+1 lives in buffer 1, the ids of tile i+2 wait in registers
+      // for the top of the next iteration, as after a generic iteration)
+      int sbu;
+      if (i + 1 < n) {
+        const int kk = min(tile_at(i + 1, sbu) * kDqKeyTile + tid, a.Lk - 1);
+        s_seg[1][tid] = kv_seg ? kv_seg[kk] : 0;
+        s_pre[1][tid] = kv_pre ? kv_pre[kk] : 0;
+      }
+      if (i + 2 < n) {
+        const int kk = min(tile_at(i + 2, sbu) * kDqKeyTile + tid, a.Lk - 1);
+        if (kv_seg) seg_r = kv_seg[kk];
+        if (kv_pre) pre_r = kv_pre[kk];
+      }
     }
   }
   for (; i < n; i += 6) {

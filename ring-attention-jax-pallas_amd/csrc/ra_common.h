@@ -337,6 +337,31 @@ RA_DEV void query_tile_range(int flags, int window, int klo, int khi, int q_off,
   lo = min(max(lo, 0), hi);
 }
 
+// Smallest and largest id of tile t (T tokens) of an id array of length L.  The loads are
+// independent of each other and issued together (a loop with a data-dependent bound would wait
+// for each load in turn: tens of microseconds per tile).
+template <int T>
+RA_DEV void tile_id_range(const int* ids, int t, int L, int& mn, int& mx) {
+  mn = 0x7fffffff;
+  mx = (int)0x80000000;
+  const int base = t * T;
+  if (base + T <= L && (((unsigned long long)(ids + base)) & 15ull) == 0) {
+#pragma unroll 4
+    for (int c = 0; c < T / 4; ++c) {
+      const i32x4 v = *(const i32x4*)(ids + base + 4 * c);
+      mn = min(min(mn, v[0]), min(v[1], min(v[2], v[3])));
+      mx = max(max(mx, v[0]), max(v[1], max(v[2], v[3])));
+    }
+  } else {
+#pragma unroll 8
+    for (int e = 0; e < T; ++e) {
+      const int sid = ids[min(base + e, L - 1)];  // repeats of the last id change nothing
+      mn = min(mn, sid);
+      mx = max(mx, sid);
+    }
+  }
+}
+
 // Executed by ONE wave.  `list` holds `cnt` entries (tile index in bits 0..14, bit 15 set when
 // the tile needs the elementwise segment test).  Finds the first run of entries that need no test
 // and whose tile indices are consecutive: ordinals [start, end), and `tile_base` such that entry

@@ -142,13 +142,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       qmax = max(qmax, s_red[8 + w]);
     }
     for (int j = j_lo + tid; j < j_hi; j += kFwdThreads) {
-      int kmin = 0x7fffffff, kmax = (int)0x80000000;
-      const int kend = min((j + 1) * kKeyTile, a.Lk);
-      for (int kk = j * kKeyTile; kk < kend; ++kk) {
-        int sid = kv_seg[kk];
-        kmin = min(kmin, sid);
-        kmax = max(kmax, sid);
-      }
+      int kmin, kmax;
+      tile_id_range<kKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
       const bool act = !(kmax < qmin || kmin > qmax);
       const bool uniform = (kmin == kmax) && (qmin == qmax) && (kmin == qmin);
       s_flag[j - j_lo] = act ? (uniform ? 1 : 3) : 0;
