@@ -104,6 +104,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   const int wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
+  RA_STAMP(0);
   const int nkt = (a.Lk + KEYS_WG - 1) / KEYS_WG;
   int hh, kt;
   decode_block(blockIdx.x, a.B * a.H, nkt, hh, kt);
@@ -156,6 +157,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     }
   }
 
+  RA_STAMP(1);
   // ---- which query tiles does this workgroup visit -------------------------------------------
   const int ntiles = (a.Lq + kQTile - 1) / kQTile;
   const int k_hi = min(k0 + KEYS_WG, a.Lk) - 1;
@@ -425,7 +427,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (n > 0) issue_tile(tile_at(0, sbu), 0, xr[0]);
     if (n > 1) issue_tile(tile_at(1, sbu), 1, xr[1]);
     if (n > 2) issue_tile(tile_at(2, sbu), 2, xr[2]);  // its statistics are stored in iteration 1
+    RA_STAMP(2);
     __builtin_amdgcn_s_waitcnt(0);
+    RA_STAMP(3);
     if (n > 0) store_stat(0, xr[0]);
     if (n > 1) store_stat(1, xr[1]);
   }
@@ -455,6 +459,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       if (needs_bias(qt0, segbit, cls)) prepare(s_c, qt0, segbit, cls, 0);
     }
   }
+  RA_STAMP(4);
   // P(i-1) and dS(i-1), packed in pairs, waiting for their dV / dK products
   u32x4 pfw[2], dsw[2];
 #pragma unroll
@@ -708,6 +713,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     if (i + 4 < n) iteration(P4{}, i + 4);
     if (i + 5 < n) iteration(P5{}, i + 5);
   }
+  RA_STAMP(5);
   if (pend_valid) {  // products of the last tile
     bf16x8 pf[2], dsf[2];
 #pragma unroll
@@ -720,6 +726,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   }
 
   RA_PROF_DUMP;
+  RA_STAMP(6);
   // ---- accumulate into the fp32 gradients owned by this key slab ------------------------------
   // All loads of an array are issued before the first value is needed: a load - add - store chain
   // per element would cost one memory round trip each, a hundred in a row with nothing to hide them.
@@ -753,6 +760,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     add_to(dkp, dk, a.sm_scale);
     add_to(dvp, dv, 1.0f);
   }
+  RA_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -780,6 +788,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   constexpr int TILE_BYTES = kDqKeyTile * ROWB;
   constexpr int NBUF = 6;
 
+  RA_STAMP(0);
   __shared__ __attribute__((aligned(16))) char s_k[NBUF][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char s_v[NBUF][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) int s_seg[NBUF][kDqKeyTile];
@@ -1061,8 +1070,10 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     }
     if (n > 2) issue_tile(tile_at(2, sbu), 2);  // its ids are stored at the top of iteration 0
   }
+  RA_STAMP(2);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
+  RA_STAMP(3);
 
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
@@ -1093,6 +1104,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       if (cur_scaled) prepare(s_a, kt0, segbit, cls, 0);
     }
   }
+  RA_STAMP(4);
   // dS^T(i-1), packed in pairs, waiting for its dQ^T product
   u32x4 dsw[2];
 #pragma unroll
@@ -1300,6 +1312,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
+  RA_STAMP(5);
   if (pend_valid) {  // product of the last tile
     bf16x8 dsf[2];
     dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
@@ -1308,6 +1321,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   }
 
   RA_PROFQ_DUMP;
+  RA_STAMP(6);
   if (q_valid) {
     float* dq = a.dq + row * D + 4 * g;
 #pragma unroll
@@ -1320,6 +1334,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
         *(f32x4*)(dq + 32 * db + 8 * bb) = t;
       }
   }
+  RA_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------

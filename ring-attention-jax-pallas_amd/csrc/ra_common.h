@@ -43,6 +43,18 @@ __device__ unsigned int g_prof[2][16];
 #define RA_PROF_DUMP do { } while (0)
 #endif
 
+// Optional wall-clock stamps of one workgroup in the middle of the grid (build with -DRA_STAMPS):
+// g_stamp[k] receives the 100 MHz counter when thread 0 of that workgroup passes RA_STAMP(k).
+#ifdef RA_STAMPS
+__device__ unsigned long long g_stamp[16];
+#define RA_STAMP(k)                                                                           \
+  do {                                                                                        \
+    if (threadIdx.x == 0 && blockIdx.x == gridDim.x / 2) g_stamp[k] = wall_clock64();         \
+  } while (0)
+#else
+#define RA_STAMP(k) do { } while (0)
+#endif
+
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 #define RA_NEG_INF (-__builtin_inff())

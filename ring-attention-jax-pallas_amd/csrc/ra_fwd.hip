@@ -59,6 +59,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     s_clock[1] = wall_clock64();
   }
 #endif
+  RA_STAMP(0);
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   int hh, qt;
   decode_block(blockIdx.x, a.B * a.H, nqt, hh, qt);
@@ -113,6 +114,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.kv_seg + b * bs.kv_seg_sb : nullptr;
   const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.kv_pre + b * bs.kv_pre_sb : nullptr;
 
+  RA_STAMP(1);
   // ---- which key tiles does this workgroup visit ------------------------------------------
   const int ntiles = (a.Lk + kKeyTile - 1) / kKeyTile;
   const int q_rows_hi = min(q0 + kFwdRows, a.Lq) - 1;
@@ -297,6 +299,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   // barrier k the tiles K_{k+1}, V_{k-1} (late waves) and V_k are read while K_{k+2}, K_{k+3},
   // V_{k+1}, V_{k+2} land: three K and four V tiles are live.
   const bool wave_on = qw < a.Lq;
+  RA_STAMP(2);
   // what barriers -3, -2, -1 would have requested
   if (n > 0) {
     issue_k(tile_at(0, sb_unused), 0);
@@ -312,8 +315,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     issue_k(tile_at(2, sb_unused), 2);
     store_ids(2);
   }
+  RA_STAMP(3);
   __builtin_amdgcn_s_waitcnt(0);  // tiles, carry and Q operands have landed
   __syncthreads();
+  RA_STAMP(4);
 
   float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
   RA_PROF_DECL
@@ -839,7 +844,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
     if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
   }
+  RA_STAMP(5);
   if (!late_half) sync(n);  // both halves pass the same number of barriers
+  RA_STAMP(6);
 
   RA_PROF_DUMP;
 #ifdef RA_CLOCK
@@ -881,6 +888,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       }
     }
   }
+  RA_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------
