@@ -119,9 +119,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   // ---- resident key-side operands ----------------------------------------------------------
   // K is scaled once, here, so that the score MFMAs deliver S * sm_scale * log2(e) directly;
   // its rounding to bf16 perturbs a probability by a few 1e-3 relative, like the rounding of P.
-  bf16x8 kf[KS], vf[KS];
+  // They live in accumulation registers (the matrix unit reads its B operand from either file),
+  // which leaves the vector registers to the score pipeline.
+  u32x4 kfa[KS], vfa[KS];
   int k_seg = 0, k_pre = 0;
   {
+    bf16x8 kf[KS], vf[KS];
     const int ki = min(kw + l32, a.Lk - 1);
     const bf16_t* kp = a.k.ptr + b * a.k.sb + h * a.k.sh + (long long)ki * a.k.sl + 8 * g;
     const bf16_t* vp = a.v.ptr + b * a.v.sb + h * a.v.sh + (long long)ki * a.v.sl + 8 * g;
@@ -134,7 +137,23 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     }
     if (GENERAL && (flags & RA_BIAS_SEGMENT)) k_seg = bs.kv_seg[b * bs.kv_seg_sb + ki];
     if (GENERAL && (flags & RA_BIAS_PREFIX)) k_pre = bs.kv_pre[b * bs.kv_pre_sb + ki];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      // an empty statement whose result is bound to accumulation registers: the compiler
+      // copies the four words there, and the fragment stays one aligned register tuple
+      asm volatile("" : "=a"(kfa[s]) : "0"(__builtin_bit_cast(u32x4, kf[s])));
+      asm volatile("" : "=a"(vfa[s]) : "0"(__builtin_bit_cast(u32x4, vf[s])));
+    }
   }
+  // acc += A x B with the accumulator in VECTOR registers and B in accumulation registers.  The
+  // compiler gives every matrix instruction of a kernel the same register class for its result;
+  // this kernel wants dK / dV in accumulation registers for the whole loop and the score tiles in
+  // vector registers, where the vector ALU reads them without a copy, hence the assembly.  No
+  // instruction depends on the result for hundreds of cycles (the next use of a score tile is
+  // one iteration away; chained accumulations alternate between two tiles).
+  auto mfma_scores = [&](f32x16& acc, const bf16x8& av, const u32x4& b_acc) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "a"(b_acc));
+  };
   float slope2 = 0.f;
   if (GENERAL && (flags & RA_BIAS_ALIBI)) slope2 = bs.slopes[h] * kLog2e;
   const int* q_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.q_seg + b * bs.q_seg_sb : nullptr;
@@ -359,14 +378,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   // S * scale2 - lse2 = Q K'^T and dP - delta = dO V^T of one tile, nothing interleaved
   auto compute_s_dp = [&](f32x16& S, f32x16& P, const char* qt, const char* dot, int buf) {
     bf16x8 fr[2 * KS];
-    f32x16 cS, cP;
 #pragma unroll
     for (int bb = 0; bb < 4; ++bb) {
       const f32x4 t0 = stat_chunk(buf, 0, bb), t1 = stat_chunk(buf, 1, bb);
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
-        cS[4 * bb + c] = t0[c];
-        cP[4 * bb + c] = t1[c];
+        S[4 * bb + c] = t0[c];
+        P[4 * bb + c] = t1[c];
       }
     }
 #pragma unroll
@@ -375,8 +393,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PFN < 2 * KS) fr[op + PFN] = nat_frag(((op + PFN) & 1) ? dot : qt, (op + PFN) >> 1);
-      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], vf[op >> 1], op == 1 ? cP : P, 0, 0, 0);
-      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], kf[op >> 1], op == 0 ? cS : S, 0, 0, 0);
+      if (op & 1) mfma_scores(P, fr[op], vfa[op >> 1]);
+      else mfma_scores(S, fr[op], kfa[op >> 1]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -448,15 +466,18 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);
   plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
 
-  f32x16 s_c, p_c;  // S(i) * scale2 - lse2 and dP(i) - delta of the current tile
+  // S(i) * scale2 - lse2 and dP(i) - delta of the current tile, in vector registers: the pair
+  // (s_a, p_a) for even i, (s_b, p_b) for odd i; an iteration consumes one pair while the matrix
+  // unit fills the other
+  f32x16 s_a, p_a, s_b, p_b;
   bool cur_valid = false;
   if (n > 0 && wave_on) {
     int qt0, segbit;
     const int cls = tile_class(0, qt0, segbit);
     if (!(cls & 1)) {
       cur_valid = true;
-      compute_s_dp(s_c, p_c, s_q[0], s_do[0], 0);
-      if (needs_bias(qt0, segbit, cls)) prepare(s_c, qt0, segbit, cls, 0);
+      compute_s_dp(s_a, p_a, s_q[0], s_do[0], 0);
+      if (needs_bias(qt0, segbit, cls)) prepare(s_a, qt0, segbit, cls, 0);
     }
   }
   RA_STAMP(4);
@@ -474,7 +495,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 
   RA_PROF_DECL
   // Generic iteration.  Tile j lives in LDS buffer j % NB = PH for j = i.
-  auto iteration = [&](auto phase, int i) {
+  auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
     constexpr int PHP = (PH + NB - 1) % NB, PH1 = (PH + 1) % NB, PH2 = (PH + 2) % NB, PH3 = (PH + 3) % NB;
     // this wave's share of tile i+1 is in LDS once at most the loads of tile i+2 are in flight;
@@ -506,8 +527,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
         float p[2], ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          p[e] = fast_exp2(s_c[r + e]);
-          ds[e] = p[e] * p_c[r + e];
+          p[e] = fast_exp2(SC[r + e]);
+          ds[e] = p[e] * PC[r + e];
         }
         pfw[r >> 3][(r & 7) >> 1] = pack2(p[0], p[1]);
         dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
@@ -524,9 +545,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       nxt_valid = !(ncls & 1);
     }
     if (nxt_valid) {
-      compute_s_dp(s_c, p_c, s_q[PH1], s_do[PH1], PH1);
+      compute_s_dp(SN, PN, s_q[PH1], s_do[PH1], PH1);
       if (!(i + 1 >= plain_lo && i + 1 < plain_hi) && needs_bias(nqt0, nsegbit, ncls))
-        prepare(s_c, nqt0, nsegbit, ncls, PH1);
+        prepare(SN, nqt0, nsegbit, ncls, PH1);
     }
     cur_valid = nxt_valid;
   };
@@ -546,7 +567,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 
   // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
   // exists and is complete, so there is nothing to classify and no flag to consult.
-  auto plain_iteration = [&](auto phase, int i) {
+  auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
     constexpr int PHP = (PH + NB - 1) % NB, PH1 = (PH + 1) % NB, PH2 = (PH + 2) % NB, PH3 = (PH + 3) % NB;
     const char* qp = s_q[PHP];
@@ -572,10 +593,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       dsf[ks] = __builtin_bit_cast(bf16x8, dsw[ks]);
     }
     bf16x8 fra[2 * KS];
-    float sc[16], pc[16];  // S(i), dP(i) handed to the vector ALU
-    f32x16 cS, cP;         // initial accumulator values of S(i+1), dP(i+1)
     constexpr int NOPS = 4 * DB;
-    constexpr int RPO = 32 / NOPS > 4 ? 32 / NOPS : 4;  // accumulator registers handed over per MFMA
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int op = 0; op < NOPS; ++op) {
@@ -607,22 +625,15 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
           do_run += (long long)kQTile * a.dout.sl;
         }
       }
-      // S(i), dP(i) leave the accumulation registers in the first half of the block ...
-#pragma unroll
-      for (int e = 0; e < RPO; ++e) {
-        const int x = op * RPO + e;
-        if (x < 16) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(sc[x]) : "a"(s_c[x]));
-        else if (x < 32) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(pc[x - 16]) : "a"(p_c[x - 16]));
-      }
-      // ... and the statistics of tile i+1 enter them in the second half
+      // the statistics of tile i+1 are the initial values of S(i+1), dP(i+1)
       {
         const int j = op - (NOPS - 8);
         if (j >= 0) {
           const f32x4 t = stat_chunk(PH1, j >> 2, j & 3);
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
-            if (j >> 2) cP[4 * (j & 3) + c] = t[c];
-            else cS[4 * (j & 3) + c] = t[c];
+            if (j >> 2) PN[4 * (j & 3) + c] = t[c];
+            else SN[4 * (j & 3) + c] = t[c];
           }
         }
       }
@@ -636,8 +647,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PFN < 2 * KS) fra[op + PFN] = nat_frag(((op + PFN) & 1) ? don : qn, (op + PFN) >> 1);
-      if (op & 1) p_c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], vf[op >> 1], op == 1 ? cP : p_c, 0, 0, 0);
-      else s_c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], kf[op >> 1], op == 0 ? cS : s_c, 0, 0, 0);
+      if (op & 1) mfma_scores(PN, fra[op], vfa[op >> 1]);
+      else mfma_scores(SN, fra[op], kfa[op >> 1]);
       if (op == 2 && !(RA_ABLATE_B & 32)) {
         // the per-row word of tile i+2 is the oldest load but those of its tile and of tile i+3
         RA_WAIT_VMCNT(2 * LPT - 1);
@@ -648,11 +659,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
         for (int e = 0; e < EPO; ++e) {
           const int r = op * EPO + e;
           if (r < 16) {
-            pe[r] = fast_exp2(sc[r]);
+            pe[r] = fast_exp2(SC[r]);
             asm volatile("" : "+v"(pe[r]));
           }
           if (r >= 1 && r <= 16) {
-            de[r - 1] = pe[r - 1] * pc[r - 1];
+            de[r - 1] = pe[r - 1] * PC[r - 1];
             asm volatile("" : "+v"(de[r - 1]));
           }
           if (r >= 2 && r <= 16 && !(r & 1)) {
@@ -666,7 +677,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
     if (!(RA_ABLATE_B & 8)) {
-      de[15] = pe[15] * pc[15];
+      de[15] = pe[15] * PC[15];
       pfw[1][3] = pack2(pe[14], pe[15]);
       dsw[1][3] = pack2(de[14], de[15]);
     }
@@ -687,31 +698,31 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
       DENSE ? -1 : min(min(plain_hi - 1, run_hi - 3), a.Lq / kQTile - tile_base - 3));
   int i = 0;
   for (; i < n && !(i > plain_lo && i + NB <= plain_end); i += NB) {
-    iteration(P0{}, i);
-    if (i + 1 < n) iteration(P1{}, i + 1);
-    if (i + 2 < n) iteration(P2{}, i + 2);
-    if (i + 3 < n) iteration(P3{}, i + 3);
-    if (i + 4 < n) iteration(P4{}, i + 4);
-    if (i + 5 < n) iteration(P5{}, i + 5);
+    iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+    if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+    if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
   if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
     if (i + NB <= plain_end) seek_plain(tile_base + i + 3);
     for (; i + NB <= plain_end; i += NB) {
-      plain_iteration(P0{}, i);
-      plain_iteration(P1{}, i + 1);
-      plain_iteration(P2{}, i + 2);
-      plain_iteration(P3{}, i + 3);
-      plain_iteration(P4{}, i + 4);
-      plain_iteration(P5{}, i + 5);
+      plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
+      plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+      plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+      plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+      plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+      plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
     }
   }
   for (; i < n; i += NB) {
-    iteration(P0{}, i);
-    if (i + 1 < n) iteration(P1{}, i + 1);
-    if (i + 2 < n) iteration(P2{}, i + 2);
-    if (i + 3 < n) iteration(P3{}, i + 3);
-    if (i + 4 < n) iteration(P4{}, i + 4);
-    if (i + 5 < n) iteration(P5{}, i + 5);
+    iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    if (i + 2 < n) iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    if (i + 3 < n) iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+    if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+    if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
   RA_STAMP(5);
   if (pend_valid) {  // products of the last tile
