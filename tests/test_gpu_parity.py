@@ -1,5 +1,5 @@
 """GPU parity tests: the HIP kernels (through the C ABI) against the CPU oracle on the same
-seeded inputs.  Tolerances are BASELINE's: forward output max-abs error <= 1e-2 and
+seeded inputs.  Tolerances: forward output max-abs error <= 1e-2 and
 logsumexp <= 1e-3 for bf16 inputs against the fp64 oracle on the same bf16-rounded values,
 dq/dk/dv relative error <= 2e-2 (max|diff| / max|ref| and Frobenius)."""
 import glob
@@ -107,7 +107,7 @@ def test_reference_shapes_self_attention(device, seed, length, h, d):
 
 # ---- bias functors --------------------------------------------------------------------------------
 def test_causal_c1_config(device):
-    # BASELINE config 1: B=1 H=4 S=1024 D=64, ring of 4 shards of 256, causal
+    # benchmark config 1: B=1 H=4 S=1024 D=64, ring of 4 shards of 256, causal
     _check(device, "C1", 1, 1024, 1024, 4, 64, 4, ra.causal_bias(), R.make_bias_fn(causal=True))
 
 
@@ -409,7 +409,7 @@ def test_fp32_and_fp16_inputs_are_cast(device):
     assert np.abs(out_bf.float().cpu().numpy() - want).max() <= 2e-2  # bf16 output rounding on top
 
 
-# ---- BASELINE configs at full size -------------------------------------------------------------------------
+# ---- benchmark configs at full size -------------------------------------------------------------------------
 def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, bias_col, qkw=None, kvkw=None):
     """Full-size run on the GPU; the oracle is evaluated densely (fp64) on sampled query rows
     (out, lse, dq) and sampled key columns (dk, dv; these use the GPU's lse/out for the other
