@@ -807,6 +807,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ int s_red[20];
+  __shared__ float s_rowc[2][kDqThreads];
   // The GENERAL variants are a few registers short in their straight-line loop: the first operand
   // fragments of Q and dO and the per-lane load offsets wait here and are fetched once per
   // iteration instead (a spill to scratch memory would make every iteration wait for all loads).
@@ -837,7 +838,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     const bf16_t* dp = a.dout.ptr + b * a.dout.sb + h * a.dout.sh + (long long)qi_c * a.dout.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      qf[s] = *(const bf16x8*)(qp + 16 * s);
+      // Q is scaled once, here, so that the score MFMAs deliver S * sm_scale * log2(e) directly
+      // (its rounding to bf16 perturbs a probability by a few 1e-3 relative, like the rounding
+      // of P; dQ itself is built from the unscaled K)
+      const bf16x8 qr = *(const bf16x8*)(qp + 16 * s);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qf[s][e] = (bf16_t)((float)qr[e] * a.scale2);
       dof[s] = *(const bf16x8*)(dp + 16 * s);
     }
     if (GENERAL) {
@@ -847,8 +853,13 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   }
   const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
   const float Lraw = a.lse[row];
-  const float neg_lse2 = (Lraw == RA_NEG_INF) ? RA_NEG_INF : -Lraw * kLog2e;  // fully masked row: P = 0
-  const float delta = a.delta[row];
+  float neg_lse2 = (Lraw == RA_NEG_INF) ? RA_NEG_INF : -Lraw * kLog2e;  // fully masked row: P = 0
+  float delta = a.delta[row];
+  // exp2(S - lse2) (dP - delta) = exp2(S) (c dP - c delta) with c = exp2(-lse2): one vector
+  // instruction less per score.  Only where no row's logsumexp is so large that exp2(S) or c
+  // could leave the fp32 range (S <= lse2 always); other waves have no straight-line stretch.
+  const bool lse_in_range = __all(fabsf(neg_lse2) <= 100.0f);
+  float c_row = 0.f, cd_row = 0.f;
   f32x16 acc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -1060,8 +1071,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     tb.dense_vs = 1;
     const int var0 = kt0 + 4 * g;
     tb.var_limit = a.Lk - var0;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) S[r] *= a.scale2;
     const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
     if (DENSE)
       tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
@@ -1089,7 +1098,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
+  if (wave_on && lse_in_range && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
     key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
@@ -1104,15 +1113,14 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
 
   f32x16 s_a, p_a, s_b, p_b;
-  bool cur_valid = false, cur_scaled = false;
+  bool cur_valid = false;
   if (n > 0 && wave_on) {
     int kt0, segbit;
     const int cls = tile_class(0, kt0, segbit);
     if (!(cls & 1)) {
       cur_valid = true;
       compute_s_dp(s_a, p_a, s_k[0], s_v[0]);
-      cur_scaled = needs_bias(kt0, segbit, cls);
-      if (cur_scaled) prepare(s_a, kt0, segbit, cls, 0);
+      if (needs_bias(kt0, segbit, cls)) prepare(s_a, kt0, segbit, cls, 0);
     }
   }
   RA_STAMP(4);
@@ -1149,13 +1157,13 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       compute_dq(dsf, s_k[PHP]);
     }
     int nkt0 = 0, nsegbit = 0, ncls = 1;
-    bool nxt_valid = false, nxt_scaled = false;
+    bool nxt_valid = false, nxt_bias = false;
     if (i + 1 >= plain_lo && i + 1 < plain_hi) {
       nxt_valid = true;
     } else if (i + 1 < n && wave_on) {
       ncls = tile_class(i + 1, nkt0, nsegbit);
       nxt_valid = !(ncls & 1);
-      nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
+      nxt_bias = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
     }
     if (nxt_valid) compute_s_dp(SN, PN, s_k[PH1], s_v[PH1]);
     if (cur_valid) {
@@ -1164,16 +1172,14 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
         float ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          const float t = cur_scaled ? SC[r + e] + neg_lse2 : fmaf(SC[r + e], a.scale2, neg_lse2);
-          ds[e] = fast_exp2(t) * (PC[r + e] - delta);
+          ds[e] = fast_exp2(SC[r + e] + neg_lse2) * (PC[r + e] - delta);
         }
         dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
       }
     }
     pend_valid = cur_valid;
-    if (nxt_scaled) prepare(SN, nkt0, nsegbit, ncls, PH1);
+    if (nxt_bias) prepare(SN, nkt0, nsegbit, ncls, PH1);
     cur_valid = nxt_valid;
-    cur_scaled = nxt_scaled;
   };
 
   // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
@@ -1252,7 +1258,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
 #pragma unroll
         for (int e = 0; e < EPO; ++e) {
           const int r = op * EPO + e;
-          float ds = fast_exp2(fmaf(SC[r], a.scale2, neg_lse2)) * (PC[r] - delta);
+          float ds = fast_exp2(SC[r]) * fmaf(PC[r], c_row, cd_row);
           asm volatile("" : "+v"(ds));  // pins the arithmetic between two MFMAs
           if (r & 1) {
             unsigned dw = pack2(ds_prev, ds);
@@ -1290,6 +1296,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
     const bool stretch = i + 6 <= plain_end;
     if (GENERAL && stretch) seg_r = pre_r = 0;  // stored already; not carried through the stretch
+    if (stretch) {
+      // the two row constants of the stretch replace the two of the generic iterations, which
+      // wait in LDS meanwhile (the kernel has no register to spare)
+      c_row = fast_exp2(neg_lse2);
+      cd_row = -c_row * delta;
+      s_rowc[0][tid] = neg_lse2;
+      s_rowc[1][tid] = delta;
+      neg_lse2 = delta = 0.f;
+    }
     for (; i + 6 <= plain_end; i += 6) {
       plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
       plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
@@ -1297,6 +1312,10 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
       plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
       plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+    }
+    if (stretch) {
+      neg_lse2 = s_rowc[0][tid];
+      delta = s_rowc[1][tid];
     }
     if (GENERAL && stretch && tid < kDqKeyTile) {
       // the stretch moved no ids: those of the two tiles in flight are fetched now (i is a
