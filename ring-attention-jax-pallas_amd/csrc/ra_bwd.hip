@@ -1239,7 +1239,39 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       q0 = s_q0[tid];
       do0 = s_do0[tid];
     }
-    float ds_prev = 0.f;
+    // The chain of a score element (exp2 and the scaled dP, their product, the packing of a
+    // pair) is spread over three consecutive MFMA slots, one link per slot, so that no vector
+    // instruction waits for the result of the one before it.
+    constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+    float ev[16], uv[16], dsv[16];
+    auto chain_links = [&](int slot) {
+#pragma unroll
+      for (int e = 0; e < EPO; ++e) {
+        const int r = slot * EPO + e;
+        if (r >= 0 && r < 16) {
+          ev[r] = fast_exp2(SC[r]);
+          uv[r] = fmaf(PC[r], c_row, cd_row);
+          asm volatile("" : "+v"(ev[r]), "+v"(uv[r]));  // pins the arithmetic between two MFMAs
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < EPO; ++e) {
+        const int r = (slot - 1) * EPO + e;
+        if (r >= 0 && r < 16) {
+          dsv[r] = ev[r] * uv[r];
+          asm volatile("" : "+v"(dsv[r]));
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < EPO; ++e) {
+        const int r = (slot - 2) * EPO + e;
+        if (r >= 0 && r < 16 && (r & 1)) {
+          unsigned dw = pack2(dsv[r - 1], dsv[r]);
+          asm volatile("" : "+v"(dw));
+          dsw[r >> 3][(r & 7) >> 1] = dw;
+        }
+      }
+    };
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PF < 2 * KS) fra[op + PF] = nat_frag(((op + PF) & 1) ? vn : kn, (op + PF) >> 1);
@@ -1253,23 +1285,11 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
         if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], dof[op >> 1], PN, 0, 0, 0);
         else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], qf[op >> 1], SN, 0, 0, 0);
       }
-      constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
-      if (op * EPO < 16) {
-#pragma unroll
-        for (int e = 0; e < EPO; ++e) {
-          const int r = op * EPO + e;
-          float ds = fast_exp2(SC[r]) * fmaf(PC[r], c_row, cd_row);
-          asm volatile("" : "+v"(ds));  // pins the arithmetic between two MFMAs
-          if (r & 1) {
-            unsigned dw = pack2(ds_prev, ds);
-            asm volatile("" : "+v"(dw));
-            dsw[r >> 3][(r & 7) >> 1] = dw;
-          }
-          ds_prev = ds;
-        }
-      }
+      chain_links(op);
       __builtin_amdgcn_sched_barrier(0);
     }
+    chain_links(2 * KS);      // the links that the last slots left over
+    chain_links(2 * KS + 1);
     RA_PROFQ_MARK(i, 4);
   };
 
