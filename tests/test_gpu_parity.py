@@ -367,6 +367,35 @@ def test_block_api_dense_bias(device):
         ra.fwd_block(tq, tk, tv, tb[:, :, :, :-1], o, m, l, scale)
 
 
+def test_dense_bias_adds_to_declarative_terms(device):
+    """A dense block and the in-kernel terms add up (here: a finite dense bias over a causal mask
+    with shard offsets), forward and backward, through the block API."""
+    B, H, Lq, Lk, D = 1, 2, 384, 256, 128
+    q, k, v, do = R.make_inputs(13, B, Lq, Lk, H, D)
+    rng = np.random.default_rng(13)
+    dense = rng.standard_normal((B, H, Lq, Lk)).astype(np.float32)
+    q_off, kv_off = 200, 100
+    causal = np.where((kv_off + np.arange(Lk))[None, :] <= (q_off + np.arange(Lq))[:, None], 0.0, -np.inf)
+    total = dense.astype(np.float64) + causal[None, None]
+    hq, hk, hv, hdo = (np.ascontiguousarray(np.transpose(x, (0, 2, 1, 3))) for x in (q, k, v, do))
+    tq, tk, tv, tdo = (_dev(x, device, torch.bfloat16) for x in (hq, hk, hv, hdo))
+    bias = ra.BlockBias(ra.causal_bias(), q_offset=q_off, kv_offset=kv_off, dense=_dev(dense, device))
+    o, m, l = rr.init_carry(B, H, Lq, D, device)
+    scale = 1 / math.sqrt(D)
+    o, m, l = ra.fwd_block(tq, tk, tv, bias, o, m, l, scale)
+    f64 = lambda x: x.astype(np.float64)
+    wo, wm, wl = R.fwd_block(f64(hq), f64(hk), f64(hv), total, np.zeros((B, H, Lq, D)),
+                             np.full((B, H, Lq), -np.inf), np.zeros((B, H, Lq)), scale)
+    assert np.abs(m.cpu().numpy() - wm).max() <= 1e-4
+    assert np.abs((o / l[..., None]).cpu().numpy() - wo / wl[..., None]).max() <= OUT_TOL
+    dq, dk, dv = ra.bwd_block(tq, tk, tv, bias, o / l[..., None], m + torch.log(l), tdo, scale)
+    wdq, wdk, wdv = R.bwd_block(f64(hq), f64(hk), f64(hv), total, wo / wl[..., None], wm + np.log(wl),
+                                f64(hdo), scale)
+    for got, ref in ((dq, wdq), (dk, wdk), (dv, wdv)):
+        mx, fro = _rel(got.cpu().numpy(), ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL
+
+
 def test_delta_kernel(device):
     B, H, L, D = 2, 3, 100, 64
     rng = np.random.default_rng(0)
