@@ -150,6 +150,9 @@ def main():
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--workload", default="C3b", choices=sorted(WORKLOADS))
+    ap.add_argument("--impl", default="hip", choices=["hip", "hip_fused"],
+                    help="hip: one launch per ring step (the headline); hip_fused: one launch per ring pass, "
+                         "the kernels walk the shards themselves (no per-kernel roofline in that mode)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
@@ -225,13 +228,19 @@ def main():
 
     ev = lambda: torch.cuda.Event(enable_timing=True)
 
+    fused = args.impl == "hip_fused"
+    ring_fwd = rr._ring_forward_fused if fused else rr._ring_forward
+    ring_bwd = rr._ring_backward_fused if fused else rr._ring_backward
+    if fused:
+        args.no_kernel_timing = True
+
     def one_step(marks=None):
         if marks is not None:
             marks[0].record()
-        out, lse = rr._ring_forward(q, k, v, plan, sm_scale, torch.bfloat16)
+        out, lse = ring_fwd(q, k, v, plan, sm_scale, torch.bfloat16)
         if marks is not None:
             marks[1].record()
-        grads = rr._ring_backward(q, k, v, out, lse, do, plan, sm_scale)
+        grads = ring_bwd(q, k, v, out, lse, do, plan, sm_scale)
         if marks is not None:
             marks[2].record()
         return out, grads
@@ -256,7 +265,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}", "B": B, "H": H, "D": D, "S": S,
-                   "ring_size": n, "bias": w["bias"], "unmasked_pairs_per_head": P},
+                   "ring_size": n, "bias": w["bias"], "unmasked_pairs_per_head": P,
+                   "launches": "one per ring pass" if fused else "one per ring step"},
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "fwd": {"ms": round(fwd_ms, 3), "tflops": round(flops_fwd / fwd_ms / 1e9, 2),
                 "pct_of_bf16_peak": round(100.0 * flops_fwd / fwd_ms / 1e9 / PEAK_BF16_TFLOPS, 2)},

@@ -162,6 +162,29 @@ int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t o
                     int64_t out_stride_l, int32_t B, int32_t H, int32_t L, int32_t D,
                     void* stream);
 
+/* Several ring steps in ONE launch.  steps[0 .. n_steps) are the parameter blocks that the
+ * caller would hand to ra_fwd_step / ra_bwd_step one after another, in that order; the result
+ * is the same up to the rounding of fp32 sums.  What runs differently: the kernel walks the
+ * shards itself and keeps its running state (the forward step's output and softmax statistics,
+ * dQ, or dK and dV) in registers between them, so the carry or gradient accumulator is read and
+ * written once per launch instead of once per step, and small shards cost one launch instead
+ * of one per step.  It is the loop of the reference around its block functions
+ * (ring.py:104-132 forward, ring.py:183-206 backward) for callers that hold several shards in
+ * memory at once - an emulated ring on one GPU, or a ring whose next shards have already
+ * arrived.  Steps whose scores are all masked (ra_step_is_skippable) are dropped; more than 16
+ * remaining steps are split into several launches.
+ *  - ra_fwd_steps and ra_bwd_dq_steps: one query shard against several key/value shards.  The
+ *    blocks must agree in everything but k.ptr, v.ptr, bias.kv_offset, bias.kv_segment_ids,
+ *    bias.kv_prefix and bias.dense_bias (and, for the backward, dk and dv, which are not
+ *    touched): RA_ERR_SHAPE otherwise.  ra_bwd_dq_steps accumulates dq only.
+ *  - ra_bwd_dkdv_steps: one key/value shard against several query shards (the query side is
+ *    what travels in the reference's backward ring, ring.py:195).  The blocks must agree in
+ *    everything but q.ptr, dout.ptr, lse, delta, dq (not touched), bias.q_offset,
+ *    bias.q_segment_ids, bias.q_prefix and bias.dense_bias.  Accumulates dk and dv only. */
+int ra_fwd_steps(const ra_fwd_step_params* steps, int32_t n_steps, void* stream);
+int ra_bwd_dq_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream);
+int ra_bwd_dkdv_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream);
+
 /* Host-only, pure: 1 if every score of the (query shard, key/value shard) pair is masked
  * by the positional terms of `bias` (CAUSAL / WINDOW), so that the whole ring step is an
  * identity on the carry and may be skipped; 0 otherwise.  The reference runs such steps and

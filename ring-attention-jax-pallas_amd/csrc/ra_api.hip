@@ -108,11 +108,70 @@ int kernel_mode(int flags) {
 
 constexpr float kLog2eHost = 1.4426950408889634f;
 
+ra::BwdArgs to_bwd_args(const ra_bwd_step_params& p) {
+  ra::BwdArgs a;
+  a.q = to_arg(p.q);
+  a.k = to_arg(p.k);
+  a.v = to_arg(p.v);
+  a.dout = to_arg(p.dout);
+  a.lse = p.lse;
+  a.delta = p.delta;
+  a.dq = p.dq;
+  a.dk = p.dk;
+  a.dv = p.dv;
+  a.B = p.B;
+  a.H = p.H;
+  a.Lq = p.Lq;
+  a.Lk = p.Lk;
+  a.scale2 = p.sm_scale * kLog2eHost;
+  a.sm_scale = p.sm_scale;
+  a.bias = to_bias(p.bias);
+  return a;
+}
+
+bool same_dims(const ra_bwd_step_params& p, const ra_bwd_step_params& f) {
+  return p.B == f.B && p.H == f.H && p.Lq == f.Lq && p.Lk == f.Lk && p.D == f.D && p.sm_scale == f.sm_scale;
+}
+
+bool same_strides(const ra_tensor& x, const ra_tensor& y) {
+  return x.stride_b == y.stride_b && x.stride_h == y.stride_h && x.stride_l == y.stride_l;
+}
+
+// everything of a bias description that belongs to the launch or to the query shard
+bool same_q_side(const ra_bias& x, const ra_bias& y) {
+  return x.flags == y.flags && x.window == y.window && x.q_offset == y.q_offset &&
+         x.q_segment_ids == y.q_segment_ids && x.q_segment_stride_b == y.q_segment_stride_b &&
+         x.kv_segment_stride_b == y.kv_segment_stride_b && x.q_prefix == y.q_prefix &&
+         x.q_prefix_stride_b == y.q_prefix_stride_b && x.kv_prefix_stride_b == y.kv_prefix_stride_b &&
+         x.alibi_slopes == y.alibi_slopes && x.dense_stride_b == y.dense_stride_b &&
+         x.dense_stride_h == y.dense_stride_h && x.dense_stride_q == y.dense_stride_q;
+}
+
+// ... and to the key/value shard
+bool same_kv_side(const ra_bias& x, const ra_bias& y) {
+  return x.flags == y.flags && x.window == y.window && x.kv_offset == y.kv_offset &&
+         x.kv_segment_ids == y.kv_segment_ids && x.q_segment_stride_b == y.q_segment_stride_b &&
+         x.kv_segment_stride_b == y.kv_segment_stride_b && x.kv_prefix == y.kv_prefix &&
+         x.q_prefix_stride_b == y.q_prefix_stride_b && x.kv_prefix_stride_b == y.kv_prefix_stride_b &&
+         x.alibi_slopes == y.alibi_slopes && x.dense_stride_b == y.dense_stride_b &&
+         x.dense_stride_h == y.dense_stride_h && x.dense_stride_q == y.dense_stride_q;
+}
+
+void add_kv_shard(ra::KvShardList& sl, const ra_tensor& k, const ra_tensor& v, const ra_bias& b) {
+  const int i = sl.n++;
+  sl.kv_off[i] = (int)b.kv_offset;
+  sl.k[i] = (const ra::bf16_t*)k.ptr;
+  sl.v[i] = (const ra::bf16_t*)v.ptr;
+  sl.kv_seg[i] = b.kv_segment_ids;
+  sl.kv_pre[i] = b.kv_prefix;
+  sl.dense[i] = b.dense_bias;
+}
+
 }  // namespace
 
 extern "C" {
 
-int ra_version(void) { return 1001; }
+int ra_version(void) { return 1002; }
 
 const char* ra_last_error(void) { return g_err; }
 
@@ -189,6 +248,56 @@ int ra_fwd_step(const ra_fwd_step_params* p, void* stream) {
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_step launch");
 }
 
+int ra_fwd_steps(const ra_fwd_step_params* steps, int32_t n_steps, void* stream) {
+  if (n_steps < 0) return fail(RA_ERR_SHAPE, "n_steps is negative");
+  if (n_steps == 0) return RA_OK;
+  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
+  const ra_fwd_step_params& f = steps[0];
+  for (int i = 0; i < n_steps; ++i) {
+    const ra_fwd_step_params& p = steps[i];
+    int rc = ra_fwd_step_check(&p);
+    if (rc) return rc;
+    const bool same =
+        p.B == f.B && p.H == f.H && p.Lq == f.Lq && p.Lk == f.Lk && p.D == f.D && p.sm_scale == f.sm_scale &&
+        !memcmp(&p.q, &f.q, sizeof(ra_tensor)) && p.o == f.o && p.m == f.m && p.l == f.l &&
+        same_strides(p.k, f.k) && same_strides(p.v, f.v) && same_q_side(p.bias, f.bias);
+    if (!same)
+      return fail(RA_ERR_SHAPE, "steps[%d] differs from steps[0] in more than its key/value shard "
+                                "(k.ptr, v.ptr, kv_offset, kv_segment_ids, kv_prefix, dense_bias)", i);
+  }
+  ra::FwdArgs a;
+  a.q = to_arg(f.q);
+  a.k = to_arg(f.k);
+  a.v = to_arg(f.v);
+  a.o = f.o;
+  a.m = f.m;
+  a.l = f.l;
+  a.B = f.B;
+  a.H = f.H;
+  a.Lq = f.Lq;
+  a.Lk = f.Lk;
+  a.scale2 = f.sm_scale * kLog2eHost;
+  a.bias = to_bias(f.bias);
+  ra::KvShardList sl;
+  memset(&sl, 0, sizeof(sl));
+  auto flush = [&]() -> int {
+    if (sl.n == 0) return RA_OK;
+    hipError_t e = ra::launch_fwd_steps(a, sl, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
+    sl.n = 0;
+    return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_steps launch");
+  };
+  for (int i = 0; i < n_steps; ++i) {
+    const ra_fwd_step_params& p = steps[i];
+    if (ra_step_is_skippable(&p.bias, p.Lq, p.Lk)) continue;  // identity on the carry
+    add_kv_shard(sl, p.k, p.v, p.bias);
+    if (sl.n == ra::kMaxShards) {
+      int rc = flush();
+      if (rc) return rc;
+    }
+  }
+  return flush();
+}
+
 int ra_fwd_finalize(const float* o, const float* m, const float* l, void* out, int32_t out_dtype,
                     int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l, float* lse,
                     int32_t B, int32_t H, int32_t Lq, int32_t D, void* stream) {
@@ -229,25 +338,92 @@ int ra_bwd_step_parts(const ra_bwd_step_params* p, int32_t parts, void* stream) 
   if (rc) return rc;
   if (parts < 1 || parts > 3) return fail(RA_ERR_SHAPE, "parts must be 1, 2 or 3 (got %d)", parts);
   if (ra_step_is_skippable(&p->bias, p->Lq, p->Lk)) return RA_OK;  // contributes nothing
-  ra::BwdArgs a;
-  a.q = to_arg(p->q);
-  a.k = to_arg(p->k);
-  a.v = to_arg(p->v);
-  a.dout = to_arg(p->dout);
-  a.lse = p->lse;
-  a.delta = p->delta;
-  a.dq = p->dq;
-  a.dk = p->dk;
-  a.dv = p->dv;
-  a.B = p->B;
-  a.H = p->H;
-  a.Lq = p->Lq;
-  a.Lk = p->Lk;
-  a.scale2 = p->sm_scale * kLog2eHost;
-  a.sm_scale = p->sm_scale;
-  a.bias = to_bias(p->bias);
+  const ra::BwdArgs a = to_bwd_args(*p);
   hipError_t e = ra::launch_bwd_step(a, p->D, kernel_mode(p->bias.flags), parts, (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_step launch");
+}
+
+int ra_bwd_dq_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream) {
+  if (n_steps < 0) return fail(RA_ERR_SHAPE, "n_steps is negative");
+  if (n_steps == 0) return RA_OK;
+  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
+  const ra_bwd_step_params& f = steps[0];
+  for (int i = 0; i < n_steps; ++i) {
+    const ra_bwd_step_params& p = steps[i];
+    int rc = ra_bwd_step_check(&p);
+    if (rc) return rc;
+    const bool same = same_dims(p, f) && !memcmp(&p.q, &f.q, sizeof(ra_tensor)) &&
+                      !memcmp(&p.dout, &f.dout, sizeof(ra_tensor)) && p.lse == f.lse && p.delta == f.delta &&
+                      p.dq == f.dq && same_strides(p.k, f.k) && same_strides(p.v, f.v) &&
+                      same_q_side(p.bias, f.bias);
+    if (!same)
+      return fail(RA_ERR_SHAPE, "steps[%d] differs from steps[0] in more than its key/value shard "
+                                "(k.ptr, v.ptr, dk, dv, kv_offset, kv_segment_ids, kv_prefix, dense_bias)", i);
+  }
+  const ra::BwdArgs a = to_bwd_args(f);
+  ra::KvShardList sl;
+  memset(&sl, 0, sizeof(sl));
+  auto flush = [&]() -> int {
+    if (sl.n == 0) return RA_OK;
+    hipError_t e = ra::launch_bwd_dq_steps(a, sl, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
+    sl.n = 0;
+    return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_dq_steps launch");
+  };
+  for (int i = 0; i < n_steps; ++i) {
+    const ra_bwd_step_params& p = steps[i];
+    if (ra_step_is_skippable(&p.bias, p.Lq, p.Lk)) continue;  // contributes nothing
+    add_kv_shard(sl, p.k, p.v, p.bias);
+    if (sl.n == ra::kMaxShards) {
+      int rc = flush();
+      if (rc) return rc;
+    }
+  }
+  return flush();
+}
+
+int ra_bwd_dkdv_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream) {
+  if (n_steps < 0) return fail(RA_ERR_SHAPE, "n_steps is negative");
+  if (n_steps == 0) return RA_OK;
+  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
+  const ra_bwd_step_params& f = steps[0];
+  for (int i = 0; i < n_steps; ++i) {
+    const ra_bwd_step_params& p = steps[i];
+    int rc = ra_bwd_step_check(&p);
+    if (rc) return rc;
+    const bool same = same_dims(p, f) && !memcmp(&p.k, &f.k, sizeof(ra_tensor)) &&
+                      !memcmp(&p.v, &f.v, sizeof(ra_tensor)) && p.dk == f.dk && p.dv == f.dv &&
+                      same_strides(p.q, f.q) && same_strides(p.dout, f.dout) && same_kv_side(p.bias, f.bias);
+    if (!same)
+      return fail(RA_ERR_SHAPE, "steps[%d] differs from steps[0] in more than its query shard (q.ptr, "
+                                "dout.ptr, lse, delta, dq, q_offset, q_segment_ids, q_prefix, dense_bias)", i);
+  }
+  const ra::BwdArgs a = to_bwd_args(f);
+  ra::QShardList sl;
+  memset(&sl, 0, sizeof(sl));
+  auto flush = [&]() -> int {
+    if (sl.n == 0) return RA_OK;
+    hipError_t e = ra::launch_bwd_dkdv_steps(a, sl, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
+    sl.n = 0;
+    return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_dkdv_steps launch");
+  };
+  for (int i = 0; i < n_steps; ++i) {
+    const ra_bwd_step_params& p = steps[i];
+    if (ra_step_is_skippable(&p.bias, p.Lq, p.Lk)) continue;  // contributes nothing
+    const int j = sl.n++;
+    sl.q_off[j] = (int)p.bias.q_offset;
+    sl.q[j] = (const ra::bf16_t*)p.q.ptr;
+    sl.dout[j] = (const ra::bf16_t*)p.dout.ptr;
+    sl.lse[j] = p.lse;
+    sl.delta[j] = p.delta;
+    sl.q_seg[j] = p.bias.q_segment_ids;
+    sl.q_pre[j] = p.bias.q_prefix;
+    sl.dense[j] = p.bias.dense_bias;
+    if (sl.n == ra::kMaxShards) {
+      int rc = flush();
+      if (rc) return rc;
+    }
+  }
+  return flush();
 }
 
 int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t out_stride_h,

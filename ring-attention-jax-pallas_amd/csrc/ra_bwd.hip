@@ -78,8 +78,11 @@ constexpr int kQTile = 32;  // queries per LDS tile in dkdv_kernel
 // (operands visible before the barrier, so their fetch straddles it; the next tile's loads and
 // the hand-over of S(i), dP(i) to the vector ALU issue in their shadow), then the 16 MFMAs of
 // S(i+1) = Q K^T and dP(i+1) = dO V^T with the exp2 / dS arithmetic of tile i in theirs.
-template <int D, int MODE>
-__global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
+// MULTI: the launch walks the query shards of `shards` one after another (the query side of the
+// ring steps that this key/value shard takes part in); dK / dV stay in registers between them.
+template <int D, int MODE, bool MULTI>
+__global__ __launch_bounds__(256) void dkdv_kernel(
+    const BwdArgs a, const std::conditional_t<MULTI, QShardList, NoShardList> shards) {
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int NT = 256;
@@ -156,8 +159,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   };
   float slope2 = 0.f;
   if (GENERAL && (flags & RA_BIAS_ALIBI)) slope2 = bs.slopes[h] * kLog2e;
-  const int* q_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.q_seg + b * bs.q_seg_sb : nullptr;
-  const int* q_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.q_pre + b * bs.q_pre_sb : nullptr;
 
   f32x16 dk[DB], dv[DB];
   {
@@ -176,12 +177,39 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     }
   }
 
+  RA_PROF_DECL
+  // ---- one pass of everything below per query shard ------------------------------------------
+  int q_off = bs.q_off;
+  const bf16_t* q_ptr = a.q.ptr;
+  const bf16_t* do_ptr = a.dout.ptr;
+  const float* lse_ptr = a.lse;
+  const float* delta_ptr = a.delta;
+  const int* q_seg_ptr = bs.q_seg;
+  const int* q_pre_ptr = bs.q_pre;
+  const float* dense_ptr = bs.dense;
+  int n_shards = 1;
+  if constexpr (MULTI) n_shards = shards.n;
+  for (int shard = 0; shard < n_shards; ++shard) {
+  if constexpr (MULTI) {
+    q_off = shards.q_off[shard];
+    q_ptr = shards.q[shard];
+    do_ptr = shards.dout[shard];
+    lse_ptr = shards.lse[shard];
+    delta_ptr = shards.delta[shard];
+    q_seg_ptr = shards.q_seg[shard];
+    q_pre_ptr = shards.q_pre[shard];
+    dense_ptr = shards.dense[shard];
+    // other waves may still be reading the last tile of the previous shard
+    if (shard > 0) __syncthreads();
+  }
+  const int* q_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? q_seg_ptr + b * bs.q_seg_sb : nullptr;
+  const int* q_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? q_pre_ptr + b * bs.q_pre_sb : nullptr;
   RA_STAMP(1);
   // ---- which query tiles does this workgroup visit -------------------------------------------
   const int ntiles = (a.Lq + kQTile - 1) / kQTile;
   const int k_hi = min(k0 + KEYS_WG, a.Lk) - 1;
   int i_lo, i_hi;
-  query_tile_range(flags, bs.window, bs.kv_off + k0, bs.kv_off + k_hi, bs.q_off, ntiles, kQTile, i_lo, i_hi);
+  query_tile_range(flags, bs.window, bs.kv_off + k0, bs.kv_off + k_hi, q_off, ntiles, kQTile, i_lo, i_hi);
   int n_act = i_hi - i_lo;
   bool use_list = false;
   // ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` that need no segment test
@@ -256,8 +284,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   // ---- global -> LDS ---------------------------------------------------------------------------
   // every wave moves 8 of a tile's 32 rows of Q and of dO; lane l of a load instruction fills
   // physical chunk l % CPR of row l / CPR and fetches the logical chunk the XOR layout puts there
-  const bf16_t* qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
-  const bf16_t* dobase = a.dout.ptr + b * a.dout.sb + h * a.dout.sh;
+  const bf16_t* qbase = q_ptr + b * a.q.sb + h * a.q.sh;
+  const bf16_t* dobase = do_ptr + b * a.dout.sb + h * a.dout.sh;
   constexpr int CPR = D / 8;
   constexpr int RPI = 64 / CPR;
   constexpr int NLD = 8 / RPI;
@@ -282,8 +310,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   const char* st_src;
   {
     const long long rowbase = ((long long)b * a.H + h) * a.Lq;
-    const char* c0 = (const char*)(a.lse + rowbase);
-    const char* c1 = (const char*)(a.delta + rowbase);
+    const char* c0 = (const char*)(lse_ptr + rowbase);
+    const char* c1 = (const char*)(delta_ptr + rowbase);
     const char* c2 = GENERAL && q_seg ? (const char*)q_seg : c0;
     const char* c3 = GENERAL && q_pre ? (const char*)q_pre : c0;
     st_src = st_class == 0 ? c0 : (st_class == 1 ? c1 : (st_class == 2 ? c2 : c3));
@@ -365,7 +393,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   auto tile_class = [&](int i, int& qt0, int& segbit) -> int {
     qt0 = tile_at(i, segbit) * kQTile;
     if (flags & RA_BIAS_PREFIX) return 2;
-    return classify_pos(flags, bs.window, bs.q_off + qt0, bs.q_off + qt0 + kQTile - 1, bs.kv_off + kw,
+    return classify_pos(flags, bs.window, q_off + qt0, q_off + qt0 + kQTile - 1, bs.kv_off + kw,
                         bs.kv_off + kw + 31);
   };
   auto needs_bias = [&](int qt0, int segbit, int cls) -> bool {
@@ -429,10 +457,10 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     tb.dense = nullptr;
     tb.dense_vs = 1;
     tb.var_limit = a.Lq - (qt0 + 4 * g);
-    const int rel0 = (bs.q_off + qt0 + 4 * g) - (bs.kv_off + kw + l32);
+    const int rel0 = (q_off + qt0 + 4 * g) - (bs.kv_off + kw + l32);
     const int* ids = (const int*)(stat_rd + ids_buf * STAT_BYTES);
     if (DENSE) {
-      tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)(qt0 + 4 * g) * bs.dense_sq +
+      tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)(qt0 + 4 * g) * bs.dense_sq +
                  min(kw + l32, a.Lk - 1);
       tb.dense_vs = bs.dense_sq;
     }
@@ -458,7 +486,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
   int plain_lo = 0, plain_hi = 0;
   if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
-    query_tile_plain_range(flags, bs.window, bs.kv_off + kw, bs.kv_off + kw + 31, bs.q_off, a.Lq / kQTile,
+    query_tile_plain_range(flags, bs.window, bs.kv_off + kw, bs.kv_off + kw + 31, q_off, a.Lq / kQTile,
                            kQTile, lo, hi);
     plain_lo = max(lo - tile_base, run_lo);
     plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
@@ -493,7 +521,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     return __builtin_bit_cast(unsigned, t);
   };
 
-  RA_PROF_DECL
   // Generic iteration.  Tile j lives in LDS buffer j % NB = PH for j = i.
   auto iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
@@ -735,6 +762,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(const BwdArgs a) {
     const int last = (n - 1) % NB;
     compute_dkdv(pf, dsf, s_q[0] + last * TILE_BYTES, s_do[0] + last * TILE_BYTES);
   }
+  }  // query shards
 
   RA_PROF_DUMP;
   RA_STAMP(6);
@@ -789,8 +817,11 @@ constexpr int kDqKeyTile = 32; // keys per LDS tile
 // fetch.  Iteration i, after its barrier, first runs the 8 MFMAs of dQ^T for tile i-1 (operands
 // visible before the barrier, so their fetch straddles it), then the 16 MFMAs of S^T(i+1),
 // dP^T(i+1) with the exp2 / dS arithmetic of tile i in their shadow.
-template <int D, int MODE>
-__global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
+// MULTI: the launch walks the key/value shards of `shards` one after another (consecutive ring
+// steps of one query shard); dQ stays in registers between them.
+template <int D, int MODE, bool MULTI>
+__global__ __launch_bounds__(kDqThreads) void dq_kernel(
+    const BwdArgs a, const std::conditional_t<MULTI, KvShardList, NoShardList> shards) {
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;
@@ -811,9 +842,10 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   // The GENERAL variants are a few registers short in their straight-line loop: the first operand
   // fragments of Q and dO and the per-lane load offsets wait here and are fetched once per
   // iteration instead (a spill to scratch memory would make every iteration wait for all loads).
-  __shared__ __attribute__((aligned(16))) bf16x8 s_q0[GENERAL ? kDqThreads : 1];
-  __shared__ __attribute__((aligned(16))) bf16x8 s_do0[GENERAL ? kDqThreads : 1];
-  __shared__ __attribute__((aligned(8))) unsigned s_voff[GENERAL ? kDqThreads : 1][2];
+  constexpr bool TIGHT = GENERAL || MULTI;
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q0[TIGHT ? kDqThreads : 1];
+  __shared__ __attribute__((aligned(16))) bf16x8 s_do0[TIGHT ? kDqThreads : 1];
+  __shared__ __attribute__((aligned(8))) unsigned s_voff[TIGHT ? kDqThreads : 1][2];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -846,7 +878,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
       for (int e = 0; e < 8; ++e) qf[s][e] = (bf16_t)((float)qr[e] * a.scale2);
       dof[s] = *(const bf16x8*)(dp + 16 * s);
     }
-    if (GENERAL) {
+    if (TIGHT) {
       s_q0[tid] = qf[0];
       s_do0[tid] = dof[0];
     }
@@ -873,14 +905,45 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     if (flags & RA_BIAS_PREFIX) q_pre = bs.q_pre[b * bs.q_pre_sb + qi_c];
     if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e;
   }
-  const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.kv_seg + b * bs.kv_seg_sb : nullptr;
-  const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.kv_pre + b * bs.kv_pre_sb : nullptr;
+  RA_PROFQ_DECL
+  // ---- one pass of everything below per key/value shard ------------------------------------
+  int kv_off = bs.kv_off;
+  const bf16_t* k_ptr = a.k.ptr;
+  const bf16_t* v_ptr = a.v.ptr;
+  const int* kv_seg_ptr = bs.kv_seg;
+  const int* kv_pre_ptr = bs.kv_pre;
+  const float* dense_ptr = bs.dense;
+  int n_shards = 1;
+  if constexpr (MULTI) n_shards = shards.n;
+  for (int shard = 0; shard < n_shards; ++shard) {
+  if constexpr (MULTI) {
+    kv_off = shards.kv_off[shard];
+    k_ptr = shards.k[shard];
+    v_ptr = shards.v[shard];
+    kv_seg_ptr = shards.kv_seg[shard];
+    kv_pre_ptr = shards.kv_pre[shard];
+    dense_ptr = shards.dense[shard];
+    // other waves may still be reading the last K tile of the previous shard
+    if (shard > 0) __syncthreads();
+  }
+  // Everything derived from the lane number is rebuilt per shard from an opaque copy of the
+  // thread id: hoisted out of this loop it would occupy registers across the tile loops, which
+  // have none to spare.
+  int tid_shard = threadIdx.x;
+  if constexpr (MULTI) asm volatile("" : "+v"(tid_shard));
+  const int tid = tid_shard, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
+  const int qw = q0 + wave * 32;
+  const int qi = qw + l32;
+  const bool q_valid = qi < a.Lq;
+  const bool wave_on = qw < a.Lq;
+  const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? kv_seg_ptr + b * bs.kv_seg_sb : nullptr;
+  const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? kv_pre_ptr + b * bs.kv_pre_sb : nullptr;
 
   // ---- which key tiles does this workgroup visit ------------------------------------------------
   const int ntiles = (a.Lk + kDqKeyTile - 1) / kDqKeyTile;
   const int q_rows_hi = min(q0 + kDqRows, a.Lq) - 1;
   int j_lo, j_hi;
-  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, bs.kv_off, ntiles, kDqKeyTile,
+  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, kv_off, ntiles, kDqKeyTile,
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
@@ -947,8 +1010,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   };
 
   // ---- global -> LDS: every wave moves 4 of a tile's 32 rows of K and of V ---------------------
-  const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
-  const bf16_t* vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
+  const bf16_t* kbase = k_ptr + b * a.k.sb + h * a.k.sh;
+  const bf16_t* vbase = v_ptr + b * a.v.sb + h * a.v.sh;
   constexpr int CPR = D / 8;   // 16-byte chunks per row
   constexpr int RPW = 4;       // rows per wave per tile
   // D = 128: one load instruction = 4 rows; D = 64: lanes 0..31 cover the wave's 4 rows
@@ -957,7 +1020,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   const int ld_chunk = ((tile_off<D>(ld_row, lane % CPR) - ld_row * ROWB) >> 4) * 8;
   const unsigned k_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.k.sl + ld_chunk) * 2);
   const unsigned v_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.v.sl + ld_chunk) * 2);
-  if (GENERAL) {
+  if (TIGHT) {
     s_voff[tid][0] = k_voff;
     s_voff[tid][1] = v_voff;
   }
@@ -965,7 +1028,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   auto issue_tile = [&](int j, int buf, bool with_ids = true) {
     const int k0 = j * kDqKeyTile;
     unsigned kvo = k_voff, vvo = v_voff;
-    if (GENERAL && !with_ids) {  // called from the straight-line loop
+    if (TIGHT && !with_ids) {  // called from the straight-line loop
       kvo = s_voff[tid][0];
       vvo = s_voff[tid][1];
     }
@@ -1019,8 +1082,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   auto tile_class = [&](int i, int& kt0, int& segbit) -> int {
     kt0 = tile_at(i, segbit) * kDqKeyTile;
     if (flags & RA_BIAS_PREFIX) return 2;
-    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off + kt0,
-                        bs.kv_off + kt0 + kDqKeyTile - 1);
+    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off + kt0,
+                        kv_off + kt0 + kDqKeyTile - 1);
   };
   auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (kt0 + kDqKeyTile > a.Lk);
@@ -1071,9 +1134,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     tb.dense_vs = 1;
     const int var0 = kt0 + 4 * g;
     tb.var_limit = a.Lk - var0;
-    const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
+    const int rel0 = (bs.q_off + qi) - (kv_off + var0);
     if (DENSE)
-      tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
+      tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
     apply_bias<true, DENSE>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
   };
 
@@ -1100,7 +1163,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
   int plain_lo = 0, plain_hi = 0;
   if (wave_on && lse_in_range && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
-    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kDqKeyTile,
+    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
     // ordinal of tile t inside the run: t - (first tile of the run) + run_lo
     int sbu;
@@ -1136,7 +1199,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     return __builtin_bit_cast(unsigned, t);
   };
 
-  RA_PROFQ_DECL
   // Generic iteration; (SC, PC) hold S^T(i), dP^T(i); (SN, PN) receive tile i+1.  Tile j lives in
   // LDS buffer j % 6; iteration i reads tiles i-1 (transposed) and i+1, tile i stays for the next
   // iteration, tile i+2 is landing, tile i+3 is issued.
@@ -1235,7 +1297,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     }
     RA_PROFQ_MARK(i, 3);
     bf16x8 q0 = qf[0], do0 = dof[0];
-    if (GENERAL) {
+    if (TIGHT) {
       q0 = s_q0[tid];
       do0 = s_do0[tid];
     }
@@ -1369,6 +1431,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(const BwdArgs a) {
     dsf[1] = __builtin_bit_cast(bf16x8, dsw[1]);
     compute_dq(dsf, s_k[0] + ((n - 1) % NBUF) * TILE_BYTES);
   }
+  }  // key/value shards
 
   RA_PROFQ_DUMP;
   RA_STAMP(6);
@@ -1434,13 +1497,13 @@ hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStre
     const int nkt = (a.Lk + keys_wg - 1) / keys_wg;
     dim3 grid((unsigned)(a.B * a.H * nkt)), block(256);
     if (D == 128) {
-      if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<128, 2>), grid, block, 0, stream, a);
-      else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<128, 1>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dkdv_kernel<128, 0>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<128, 2, false>), grid, block, 0, stream, a, NoShardList{});
+      else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<128, 1, false>), grid, block, 0, stream, a, NoShardList{});
+      else hipLaunchKernelGGL((dkdv_kernel<128, 0, false>), grid, block, 0, stream, a, NoShardList{});
     } else {
-      if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<64, 2>), grid, block, 0, stream, a);
-      else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<64, 1>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dkdv_kernel<64, 0>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<64, 2, false>), grid, block, 0, stream, a, NoShardList{});
+      else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<64, 1, false>), grid, block, 0, stream, a, NoShardList{});
+      else hipLaunchKernelGGL((dkdv_kernel<64, 0, false>), grid, block, 0, stream, a, NoShardList{});
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
@@ -1449,14 +1512,45 @@ hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStre
     const int nqt = (a.Lq + kDqRows - 1) / kDqRows;
     dim3 grid((unsigned)(a.B * a.H * nqt)), block(kDqThreads);
     if (D == 128) {
-      if (mode == 2) hipLaunchKernelGGL((dq_kernel<128, 2>), grid, block, 0, stream, a);
-      else if (mode == 1) hipLaunchKernelGGL((dq_kernel<128, 1>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dq_kernel<128, 0>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dq_kernel<128, 2, false>), grid, block, 0, stream, a, NoShardList{});
+      else if (mode == 1) hipLaunchKernelGGL((dq_kernel<128, 1, false>), grid, block, 0, stream, a, NoShardList{});
+      else hipLaunchKernelGGL((dq_kernel<128, 0, false>), grid, block, 0, stream, a, NoShardList{});
     } else {
-      if (mode == 2) hipLaunchKernelGGL((dq_kernel<64, 2>), grid, block, 0, stream, a);
-      else if (mode == 1) hipLaunchKernelGGL((dq_kernel<64, 1>), grid, block, 0, stream, a);
-      else hipLaunchKernelGGL((dq_kernel<64, 0>), grid, block, 0, stream, a);
+      if (mode == 2) hipLaunchKernelGGL((dq_kernel<64, 2, false>), grid, block, 0, stream, a, NoShardList{});
+      else if (mode == 1) hipLaunchKernelGGL((dq_kernel<64, 1, false>), grid, block, 0, stream, a, NoShardList{});
+      else hipLaunchKernelGGL((dq_kernel<64, 0, false>), grid, block, 0, stream, a, NoShardList{});
     }
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QShardList& shards, int D, int mode, hipStream_t stream) {
+  const int keys_wg = 128;
+  const int nkt = (a.Lk + keys_wg - 1) / keys_wg;
+  dim3 grid((unsigned)(a.B * a.H * nkt)), block(256);
+  if (D == 128) {
+    if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<128, 2, true>), grid, block, 0, stream, a, shards);
+    else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<128, 1, true>), grid, block, 0, stream, a, shards);
+    else hipLaunchKernelGGL((dkdv_kernel<128, 0, true>), grid, block, 0, stream, a, shards);
+  } else {
+    if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<64, 2, true>), grid, block, 0, stream, a, shards);
+    else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<64, 1, true>), grid, block, 0, stream, a, shards);
+    else hipLaunchKernelGGL((dkdv_kernel<64, 0, true>), grid, block, 0, stream, a, shards);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream) {
+  const int nqt = (a.Lq + kDqRows - 1) / kDqRows;
+  dim3 grid((unsigned)(a.B * a.H * nqt)), block(kDqThreads);
+  if (D == 128) {
+    if (mode == 2) hipLaunchKernelGGL((dq_kernel<128, 2, true>), grid, block, 0, stream, a, shards);
+    else if (mode == 1) hipLaunchKernelGGL((dq_kernel<128, 1, true>), grid, block, 0, stream, a, shards);
+    else hipLaunchKernelGGL((dq_kernel<128, 0, true>), grid, block, 0, stream, a, shards);
+  } else {
+    if (mode == 2) hipLaunchKernelGGL((dq_kernel<64, 2, true>), grid, block, 0, stream, a, shards);
+    else if (mode == 1) hipLaunchKernelGGL((dq_kernel<64, 1, true>), grid, block, 0, stream, a, shards);
+    else hipLaunchKernelGGL((dq_kernel<64, 0, true>), grid, block, 0, stream, a, shards);
   }
   return hipGetLastError();
 }

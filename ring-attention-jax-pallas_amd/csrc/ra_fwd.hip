@@ -27,8 +27,12 @@ constexpr int kKeyTile = 64;    // keys per LDS tile
 constexpr int kMaxListTiles = 1024;
 constexpr int kPlainMinTiles = 16;  // shortest stretch of plain tiles that takes the straight-line loop
 
-template <int D, int MODE>
-__global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) {
+// MULTI: the launch walks the key/value shards of `shards` one after another (the arguments of
+// consecutive ring steps of one query shard); the step's contribution stays in registers
+// between them and meets the carry once, at the end.
+template <int D, int MODE, bool MULTI>
+__global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
+    const FwdArgs a, const std::conditional_t<MULTI, KvShardList, NoShardList> shards) {
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;  // k-steps of the QK^T contraction
@@ -43,9 +47,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
   __shared__ int s_red[24];
   __shared__ int s_stash[GENERAL ? 3 : 1][GENERAL ? kFwdThreads : 1];
-  // The GENERAL variant is four registers short in its straight-line loop: the first operand
-  // fragment of Q waits here and is fetched once per iteration instead.
-  __shared__ __attribute__((aligned(16))) bf16x8 s_q0[GENERAL ? kFwdThreads : 1];
+  // The GENERAL and MULTI variants are a few registers short in their straight-line loop: the
+  // first operand fragment of Q waits here and is fetched once per iteration instead.
+  constexpr bool TIGHT = GENERAL || MULTI;
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q0[TIGHT ? kFwdThreads : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -78,7 +83,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     const bf16_t* qp = a.q.ptr + b * a.q.sb + h * a.q.sh + (long long)qi_c * a.q.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
-    if (GENERAL) s_q0[tid] = qf[0];
+    if (TIGHT) s_q0[tid] = qf[0];
   }
   long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
   // This step accumulates its own contribution from zero and is merged with the incoming carry
@@ -111,15 +116,47 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     if (flags & RA_BIAS_PREFIX) q_pre = bs.q_pre[b * bs.q_pre_sb + qi_c];
     if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e;
   }
-  const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? bs.kv_seg + b * bs.kv_seg_sb : nullptr;
-  const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? bs.kv_pre + b * bs.kv_pre_sb : nullptr;
+  float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
+  RA_PROF_DECL
+
+  // ---- one pass of everything below per key/value shard ------------------------------------
+  int kv_off = bs.kv_off;
+  const bf16_t* k_ptr = a.k.ptr;
+  const bf16_t* v_ptr = a.v.ptr;
+  const int* kv_seg_ptr = bs.kv_seg;
+  const int* kv_pre_ptr = bs.kv_pre;
+  const float* dense_ptr = bs.dense;
+  int n_shards = 1;
+  if constexpr (MULTI) n_shards = shards.n;
+  for (int shard = 0; shard < n_shards; ++shard) {
+  if constexpr (MULTI) {
+    kv_off = shards.kv_off[shard];
+    k_ptr = shards.k[shard];
+    v_ptr = shards.v[shard];
+    kv_seg_ptr = shards.kv_seg[shard];
+    kv_pre_ptr = shards.kv_pre[shard];
+    dense_ptr = shards.dense[shard];
+    // the late waves may still be reading the last V tile of the previous shard
+    if (shard > 0) __syncthreads();
+  }
+  // Everything derived from the lane number is rebuilt per shard from an opaque copy of the
+  // thread id: hoisted out of this loop it would occupy registers across the tile loops, which
+  // have none to spare.
+  int tid_shard = threadIdx.x;
+  if constexpr (MULTI) asm volatile("" : "+v"(tid_shard));
+  const int tid = tid_shard, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, g = lane >> 5;
+  const int qw = q0 + wave * 32;
+  const int qi = qw + l32;
+  const bool q_valid = qi < a.Lq;
+  const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? kv_seg_ptr + b * bs.kv_seg_sb : nullptr;
+  const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? kv_pre_ptr + b * bs.kv_pre_sb : nullptr;
 
   RA_STAMP(1);
   // ---- which key tiles does this workgroup visit ------------------------------------------
   const int ntiles = (a.Lk + kKeyTile - 1) / kKeyTile;
   const int q_rows_hi = min(q0 + kFwdRows, a.Lq) - 1;
   int j_lo, j_hi;
-  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, bs.kv_off, ntiles, kKeyTile,
+  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, kv_off, ntiles, kKeyTile,
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
@@ -176,8 +213,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
     tile_base = s_red[19];
   }
 
-  const bf16_t* kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
-  const bf16_t* vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
+  const bf16_t* kbase = k_ptr + b * a.k.sb + h * a.k.sh;
+  const bf16_t* vbase = v_ptr + b * a.v.sb + h * a.v.sh;
   int seg_r = 0, pre_r = 0;
 
   auto tile_at = [&](int i, int& segbit) -> int {
@@ -320,16 +357,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   __syncthreads();
   RA_STAMP(4);
 
-  float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
-  RA_PROF_DECL
   constexpr int PF = 3;  // LDS operand fetches kept in flight ahead of the MFMA that uses them
 
   // positional class of this wave's 32 x 64 rectangle of tile index i
   auto tile_class = [&](int i, int& kt0, int& segbit) -> int {
     kt0 = tile_at(i, segbit) * kKeyTile;
     if (flags & RA_BIAS_PREFIX) return 2;
-    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off + kt0,
-                        bs.kv_off + kt0 + kKeyTile - 1);
+    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off + kt0,
+                        kv_off + kt0 + kKeyTile - 1);
   };
   // Per-lane LDS byte offsets of the operand fetches.  Everything that changes from one MFMA
   // to the next (tile buffer, 32-key block, 16-key step) is a multiple of 16 rows, which the
@@ -428,9 +463,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
       for (int r = 0; r < 16; ++r) S[kb][r] *= a.scale2;
       const int var0 = kt0 + 32 * kb + 4 * g;
       tb.var_limit = a.Lk - var0;
-      const int rel0 = (bs.q_off + qi) - (bs.kv_off + var0);
+      const int rel0 = (bs.q_off + qi) - (kv_off + var0);
       if (DENSE)
-        tb.dense = bs.dense + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
+        tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
       apply_bias<true, DENSE>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
                        &s_pre[ids_buf][32 * kb + 4 * g]);
 #pragma unroll
@@ -463,7 +498,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   int plain_lo = 0, plain_hi = 0;
   if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;  // tile indices
-    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, bs.kv_off, a.Lk / kKeyTile,
+    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off, a.Lk / kKeyTile,
                          kKeyTile, lo, hi);
     plain_lo = max(lo - tile_base, run_lo);
     plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
@@ -662,7 +697,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   };
   auto plain_iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
     constexpr int PAR = decltype(parity)::value;
-    constexpr int PF = GENERAL ? 2 : 3;  // the GENERAL variant has four registers less to spare
+    constexpr int PF = TIGHT ? 2 : 3;  // these variants have four registers less to spare
     RA_PROF_MARK(i, 1);
     if (!late_half) sync_plain();
     RA_PROF_MARK(i, 2);
@@ -733,7 +768,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
 #pragma unroll
       for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
       bf16x8 q0 = qf[0];
-      if (GENERAL) q0 = s_q0[tid];
+      if (TIGHT) q0 = s_q0[tid];
       links_of_slot(-1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -847,6 +882,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(const FwdArgs a) 
   RA_STAMP(5);
   if (!late_half) sync(n);  // both halves pass the same number of barriers
   RA_STAMP(6);
+  }  // key/value shards
 
   RA_PROF_DUMP;
 #ifdef RA_CLOCK
@@ -933,19 +969,28 @@ __global__ void fwd_finalize_kernel(const float* o, const float* m, const float*
 namespace ra {
 
 // mode: 0 = causal / window terms only, 1 = any of the per-tile terms, 2 = a dense bias block too
-hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream) {
+template <bool MULTI, typename Shards>
+static hipError_t launch_fwd(const FwdArgs& a, const Shards& sl, int D, int mode, hipStream_t stream) {
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   dim3 grid((unsigned)(a.B * a.H * nqt)), block(kFwdThreads);
   if (D == 128) {
-    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<128, 2>), grid, block, 0, stream, a);
-    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<128, 1>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((fwd_step_kernel<128, 0>), grid, block, 0, stream, a);
+    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<128, 2, MULTI>), grid, block, 0, stream, a, sl);
+    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<128, 1, MULTI>), grid, block, 0, stream, a, sl);
+    else hipLaunchKernelGGL((fwd_step_kernel<128, 0, MULTI>), grid, block, 0, stream, a, sl);
   } else {
-    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<64, 2>), grid, block, 0, stream, a);
-    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<64, 1>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((fwd_step_kernel<64, 0>), grid, block, 0, stream, a);
+    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<64, 2, MULTI>), grid, block, 0, stream, a, sl);
+    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<64, 1, MULTI>), grid, block, 0, stream, a, sl);
+    else hipLaunchKernelGGL((fwd_step_kernel<64, 0, MULTI>), grid, block, 0, stream, a, sl);
   }
   return hipGetLastError();
+}
+
+hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream) {
+  return launch_fwd<false>(a, NoShardList{}, D, mode, stream);
+}
+
+hipError_t launch_fwd_steps(const FwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream) {
+  return launch_fwd<true>(a, shards, D, mode, stream);
 }
 
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream) {

@@ -28,7 +28,34 @@ struct BwdArgs {
   BiasArgs bias;
 };
 
+// Per-shard arguments of a launch that walks several shards: the key/value side of consecutive
+// ring steps of one query shard (forward, dQ) ...
+constexpr int kMaxShards = 16;
+struct KvShardList {
+  int n;
+  int kv_off[kMaxShards];
+  const bf16_t* k[kMaxShards];
+  const bf16_t* v[kMaxShards];
+  const int* kv_seg[kMaxShards];
+  const int* kv_pre[kMaxShards];
+  const float* dense[kMaxShards];
+};
+// ... or the query side of the steps that one key/value shard takes part in (dK/dV).
+struct QShardList {
+  int n;
+  int q_off[kMaxShards];
+  const bf16_t* q[kMaxShards];
+  const bf16_t* dout[kMaxShards];
+  const float* lse[kMaxShards];
+  const float* delta[kMaxShards];
+  const int* q_seg[kMaxShards];
+  const int* q_pre[kMaxShards];
+  const float* dense[kMaxShards];
+};
+struct NoShardList {};
+
 hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream);
+hipError_t launch_fwd_steps(const FwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream);
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream);
 hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, void* out, int out_f32,
                                long long sb, long long sh, long long sl, float* lse, int B, int H,
@@ -37,6 +64,8 @@ hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long lon
                             TensorArg dout, float* delta, int B, int H, int Lq, int D,
                             hipStream_t stream);
 hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStream_t stream);
+hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream);
+hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QShardList& shards, int D, int mode, hipStream_t stream);
 hipError_t launch_mfma_rate(float* sink, int blocks, int iters, int random, hipStream_t stream);
 hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl,
                                int B, int H, int L, int D, hipStream_t stream);

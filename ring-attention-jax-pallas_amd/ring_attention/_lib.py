@@ -63,6 +63,7 @@ EXPORTS = {
     "ra_fwd_init": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
                               C.c_int32, C.c_void_p]),
     "ra_fwd_step": (C.c_int, [C.POINTER(RaFwdStepParams), C.c_void_p]),
+    "ra_fwd_steps": (C.c_int, [C.POINTER(RaFwdStepParams), C.c_int32, C.c_void_p]),
     "ra_fwd_finalize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
                                   C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int32,
                                   C.c_int32, C.c_int32, C.c_void_p]),
@@ -71,6 +72,8 @@ EXPORTS = {
                                C.c_int32, C.c_void_p]),
     "ra_bwd_step": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_void_p]),
     "ra_bwd_step_parts": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
+    "ra_bwd_dq_steps": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
+    "ra_bwd_dkdv_steps": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
     "ra_bwd_finalize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32,
                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "ra_step_is_skippable": (C.c_int, [C.POINTER(RaBias), C.c_int32, C.c_int32]),

@@ -35,7 +35,10 @@ import torch
 from . import _lib
 from .bias import BiasFn, BlockBias
 
-_IMPLS = ("hip", "pallas")  # "pallas" is accepted as an alias: the fused-kernel choice
+# "hip": one launch per ring step, the reference's loop; "pallas" is accepted as an alias (the
+# fused-kernel choice there).  "hip_fused": one launch per ring PASS - the kernels walk the shards
+# of a query (or key/value) shard's whole trip around the ring themselves.
+_IMPLS = ("hip", "pallas", "hip_fused")
 
 
 @dataclass(frozen=True)
@@ -118,6 +121,38 @@ def fwd_block(q, k, v, bias: Union[BlockBias, torch.Tensor, None], o, m, l, sm_s
     return o, m, l
 
 
+def _fwd_params(q, k, v, bias, o, m, l, sm_scale) -> _lib.RaFwdStepParams:
+    B, H, Lq, D = q.shape
+    p = _lib.RaFwdStepParams()
+    p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
+    p.sm_scale = float(sm_scale)
+    p.q, p.k, p.v = _view_bhld(q), _view_bhld(k), _view_bhld(v)
+    for t_ in (o, m, l):
+        if t_.dtype != torch.float32 or not t_.is_contiguous():
+            raise ValueError("o, m, l carries must be contiguous float32 tensors")
+    p.o, p.m, p.l = o.data_ptr(), m.data_ptr(), l.data_ptr()
+    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
+    return p
+
+
+def fwd_blocks(q, kvs, biases, o, m, l, sm_scale: float):
+    """Several consecutive ring steps of one query shard in ONE launch: equivalent to
+    ``fwd_block(q, k, v, bias, o, m, l, sm_scale)`` for every ``(k, v)`` of ``kvs`` with the bias
+    of the same index, in that order (the loop ring.py:104-132), with the step's running state
+    kept in registers between the shards.  The shards share their shape and strides."""
+    _require_gpu(q)
+    lib = _lib.load()
+    steps = (_lib.RaFwdStepParams * len(kvs))()
+    keep = []  # the bias structs point into tensors that must outlive the call
+    for i, ((k, v), bias) in enumerate(zip(kvs, biases)):
+        if isinstance(bias, torch.Tensor):
+            bias = BlockBias(dense=bias)
+        keep.append(bias)
+        steps[i] = _fwd_params(q, k, v, bias, o, m, l, sm_scale)
+    _lib.check("ra_fwd_steps", lib.ra_fwd_steps(steps, len(kvs), _stream()))
+    return o, m, l
+
+
 def init_carry(batch, heads, q_len, dim, device):
     """Fresh carry o = 0, l = 0, m = -inf (ring.py:124-126), fp32."""
     lib = _lib.load()
@@ -162,8 +197,7 @@ def precompute_delta(out, do, delta=None):
     return delta
 
 
-def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, parts=3):
-    lib = _lib.load()
+def _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale) -> _lib.RaBwdStepParams:
     B, H, Lq, D = q.shape
     p = _lib.RaBwdStepParams()
     p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
@@ -172,7 +206,30 @@ def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, parts=3):
     p.lse, p.delta = lse.data_ptr(), delta.data_ptr()
     p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
+    return p
+
+
+def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, parts=3):
+    lib = _lib.load()
+    p = _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale)
     _lib.check("ra_bwd_step", lib.ra_bwd_step_parts(C.byref(p), parts, _stream()))
+
+
+def _bwd_steps(which: str, step_args, sm_scale):
+    """``step_args``: one ``(q, k, v, do, lse, delta, dq, dk, dv, bias)`` tuple per ring step, as
+    for ``_bwd_step``; ``which`` is ``"dq"`` (one query shard, several key/value shards) or
+    ``"dkdv"`` (one key/value shard, several query shards).  One launch for all of them."""
+    lib = _lib.load()
+    steps = (_lib.RaBwdStepParams * len(step_args))()
+    keep = []  # the bias structs point into tensors that must outlive the call
+    for i, args in enumerate(step_args):
+        bias = args[9]
+        if isinstance(bias, torch.Tensor):
+            bias = BlockBias(dense=bias)
+        keep.append(bias)
+        steps[i] = _bwd_params(*args[:9], bias, sm_scale)
+    fn = {"dq": "ra_bwd_dq_steps", "dkdv": "ra_bwd_dkdv_steps"}[which]
+    _lib.check(fn, getattr(lib, fn)(steps, len(step_args), _stream()))
 
 
 def bwd_block(q, k, v, bias: Union[BlockBias, torch.Tensor, None], o, L, do, sm_scale: float):
@@ -350,6 +407,58 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
     return out, lse
 
 
+def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO_TIMER):
+    """``_ring_forward`` with the whole ring pass of a query shard in one launch: the kernel
+    visits the key/value shards in ring order itself."""
+    n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
+    dev = q.device
+    out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
+    lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    o, m, l = init_carry(B, H, Lq, D, dev)
+    for r in range(n):
+        if r:
+            reset_carry(o, m, l)
+        order = [(r - t) % n for t in range(n)]  # ring.py:51-55
+        with timer.span("fwd_pass", r, -1):
+            fwd_blocks(_shard_bhld(q, r, Lq), [(_shard_bhld(k, s, Lk), _shard_bhld(v, s, Lk)) for s in order],
+                       [plan.block_bias(r, s) for s in order], o, m, l, sm_scale)
+        finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
+    return out, lse
+
+
+def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
+    """``_ring_backward`` with one launch per key/value shard for dK / dV (the kernel visits the
+    query shards in the order they arrive, ring.py:195) and one per query shard for dQ."""
+    n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
+    dev = q.device
+    delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    for s in range(n):
+        precompute_delta(_shard_bhld(out, s, Lq), _shard_bhld(do, s, Lq), delta[s])
+    dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
+    dk_acc = torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)
+    dv_acc = torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+    def step(qs, ks):
+        return (_shard_bhld(q, qs, Lq), _shard_bhld(k, ks, Lk), _shard_bhld(v, ks, Lk),
+                _shard_bhld(do, qs, Lq), lse[qs], delta[qs], dq_acc[qs], dk_acc, dv_acc,
+                plan.block_bias(qs, ks))
+
+    for r in range(n):
+        dk_acc.zero_()
+        dv_acc.zero_()
+        with timer.span("bwd_dkdv_pass", -1, r):
+            _bwd_steps("dkdv", [step((r - t) % n, r) for t in range(n)], sm_scale)
+        _finalize_grad(dk_acc, _shard_bhld(dk, r, Lk))
+        _finalize_grad(dv_acc, _shard_bhld(dv, r, Lk))
+    for s in range(n):
+        # query shard s meets key/value shard r at step (r - s) mod n of device r
+        with timer.span("bwd_dq_pass", s, -1):
+            _bwd_steps("dq", [step(s, (s + t) % n) for t in range(n)], sm_scale)
+        _finalize_grad(dq_acc[s], _shard_bhld(dq, s, Lq))
+    return dq, dk, dv
+
+
 def _ring_backward(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
@@ -386,10 +495,11 @@ class _RingAttentionFn(torch.autograd.Function):
     """custom_vjp of the reference (ring.py:214-243): forward saves (q, k, v, o, L)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, plan, sm_scale, out_dtype):
-        out, lse = _ring_forward(q, k, v, plan, sm_scale, out_dtype)
+    def forward(ctx, q, k, v, plan, sm_scale, out_dtype, fused):
+        fwd = _ring_forward_fused if fused else _ring_forward
+        out, lse = fwd(q, k, v, plan, sm_scale, out_dtype)
         ctx.save_for_backward(q, k, v, out, lse)
-        ctx.plan, ctx.sm_scale = plan, sm_scale
+        ctx.plan, ctx.sm_scale, ctx.fused = plan, sm_scale, fused
         ctx.mark_non_differentiable(lse)
         return out, lse
 
@@ -397,8 +507,9 @@ class _RingAttentionFn(torch.autograd.Function):
     def backward(ctx, do, _dlse):
         q, k, v, out, lse = ctx.saved_tensors
         do = _kernel_ready(do)
-        dq, dk, dv = _ring_backward(q, k, v, out, lse, do, ctx.plan, ctx.sm_scale)
-        return dq, dk, dv, None, None, None
+        bwd = _ring_backward_fused if ctx.fused else _ring_backward
+        dq, dk, dv = bwd(q, k, v, out, lse, do, ctx.plan, ctx.sm_scale)
+        return dq, dk, dv, None, None, None, None
 
 
 def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = None, bias_q_kwargs=None,
@@ -432,7 +543,7 @@ def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable,
         q, k, v = (torch.nn.functional.pad(x, pad) for x in (q, k, v))
     q, k, v = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
     plan = _RingPlan(q, k, n, bias_fn, bias_q_kwargs, bias_kv_kwargs)
-    out, lse = _RingAttentionFn.apply(q, k, v, plan, float(sm_scale), out_dtype)
+    out, lse = _RingAttentionFn.apply(q, k, v, plan, float(sm_scale), out_dtype, block_impl == "hip_fused")
     if d_pad != d_true:
         out = out[..., :d_true]
     if in_dtype not in (torch.float32, torch.bfloat16):
@@ -456,8 +567,10 @@ def ring_attention(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = 
             for a ``BiasFn``: ``q_segment_ids``, ``q_positions``, ``q_prefix_mask`` and their
             ``kv_`` twins.
         sm_scale: softmax scale, 1/sqrt(d) if unspecified.
-        block_impl: ``"hip"`` (``"pallas"`` is accepted as an alias); anything else raises
-            ``ValueError`` as the reference does (ring.py:312).
+        block_impl: ``"hip"`` (one kernel launch per ring step; ``"pallas"`` is accepted as an
+            alias) or ``"hip_fused"`` (one launch per ring pass: the kernels walk the shards
+            themselves, which pays when shards are small); anything else raises ``ValueError`` as
+            the reference does (ring.py:312).
     Returns:
         attention output ``[b, S, h, d]``; differentiable w.r.t. q, k, v.
     """

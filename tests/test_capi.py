@@ -125,3 +125,48 @@ def test_step_is_skippable_matches_brute_force(lib, flags, window):
             if flags & 8:
                 want = 0  # prefix masks are data dependent: never skipped on the host
             assert got == want, (flags, window, q_off, kv_off)
+
+
+def _steps(make, n):
+    arr = (type(make()) * n)()
+    for i in range(n):
+        arr[i] = make()
+    return arr
+
+
+def test_multi_step_entry_points_validate_before_any_gpu_call(lib):
+    # nothing to do / bad counts
+    assert lib.ra_fwd_steps(None, 0, None) == 0
+    assert lib.ra_fwd_steps(None, 2, None) == -1
+    assert lib.ra_bwd_dq_steps(None, -1, None) == -2
+    assert lib.ra_bwd_dkdv_steps(None, 3, None) == -1
+    # every block goes through the single-step checks
+    f = _steps(_good_fwd, 3)
+    f[2].D = 96
+    assert lib.ra_fwd_steps(f, 3, None) == -3
+    # the blocks of one launch may differ in the travelling shard only
+    f = _steps(_good_fwd, 2)
+    f[1].o = 0x3000
+    assert lib.ra_fwd_steps(f, 2, None) == -2 and b"steps[1]" in lib.ra_last_error()
+    f = _steps(_good_fwd, 2)
+    f[1].k.stride_l = 512
+    assert lib.ra_fwd_steps(f, 2, None) == -2
+    f = _steps(_good_fwd, 2)
+    f[1].bias.q_offset = 64
+    assert lib.ra_fwd_steps(f, 2, None) == -2
+    b = _steps(_good_bwd, 2)
+    b[1].lse = 0x4000          # the query side is fixed in a dq launch ...
+    assert lib.ra_bwd_dq_steps(b, 2, None) == -2
+    b = _steps(_good_bwd, 2)
+    b[1].dk = 0x4000           # ... and the key/value side in a dk/dv launch
+    assert lib.ra_bwd_dkdv_steps(b, 2, None) == -2
+    b = _steps(_good_bwd, 2)
+    b[1].bias.kv_offset = 64
+    assert lib.ra_bwd_dkdv_steps(b, 2, None) == -2
+    # steps that are masked entirely are dropped on the host: nothing is launched for these
+    for arr, fn in ((_steps(_good_fwd, 2), lib.ra_fwd_steps), (_steps(_good_bwd, 2), lib.ra_bwd_dq_steps),
+                    (_steps(_good_bwd, 2), lib.ra_bwd_dkdv_steps)):
+        for p in arr:
+            p.bias.flags = _lib.RA_BIAS_CAUSAL
+            p.bias.kv_offset = 1 << 20
+        assert fn(arr, 2, None) == 0

@@ -32,12 +32,13 @@ def _rel(a, b):
             np.linalg.norm(a - b) / max(np.linalg.norm(b), 0.05 * np.sqrt(b.size)))
 
 
-def _run_hip(device, q, k, v, do, n, fn, qkw, kvkw, sm_scale=None):
+def _run_hip(device, q, k, v, do, n, fn, qkw, kvkw, sm_scale=None, impl="hip"):
     tq, tk, tv = (_dev(x, device, torch.bfloat16).requires_grad_(True) for x in (q, k, v))
     tqkw = {a: _dev(b, device) for a, b in (qkw or {}).items()} or None
     tkvkw = {a: _dev(b, device) for a, b in (kvkw or {}).items()} or None
     out, lse = ra.ring_attention_with_lse(tq, tk, tv, n, bias_fn=fn, bias_q_kwargs=tqkw,
-                                          bias_kv_kwargs=tkvkw, sm_scale=sm_scale, out_dtype=torch.float32)
+                                          bias_kv_kwargs=tkvkw, sm_scale=sm_scale, out_dtype=torch.float32,
+                                          block_impl=impl)
     grads = None
     if do is not None:
         out.backward(_dev(do, device, torch.float32))
@@ -47,10 +48,10 @@ def _run_hip(device, q, k, v, do, n, fn, qkw, kvkw, sm_scale=None):
 
 
 def _check(device, name, B, Sq, Sk, H, D, n, fn=None, ofn=None, qkw=None, kvkw=None, std=1.0, seed=0,
-           grads=True):
-    print(f"[parity] {name}: B={B} Sq={Sq} Sk={Sk} H={H} D={D} ring={n} seed={seed}", flush=True)
+           grads=True, impl="hip"):
+    print(f"[parity] {name}: B={B} Sq={Sq} Sk={Sk} H={H} D={D} ring={n} seed={seed} impl={impl}", flush=True)
     q, k, v, do = R.make_inputs(seed, B, Sq, Sk, H, D, std=std)
-    out, lse, g = _run_hip(device, q, k, v, do if grads else None, n, fn, qkw, kvkw)
+    out, lse, g = _run_hip(device, q, k, v, do if grads else None, n, fn, qkw, kvkw, impl=impl)
     oq, okv = dict(qkw or {}), dict(kvkw or {})
     bias = None
     if ofn is not None:
@@ -396,6 +397,125 @@ def test_dense_bias_adds_to_declarative_terms(device):
         assert mx <= GRAD_TOL and fro <= GRAD_TOL
 
 
+# ---- several ring steps per launch (ra_fwd_steps, ra_bwd_dq_steps, ra_bwd_dkdv_steps) -----------
+def _fused_cases():
+    seg = R.geometric_segment_ids(0, 2, 2048, 300)
+    rng = np.random.default_rng(5)
+    segr = rng.integers(0, 5, (2, 512)).astype(np.int32)
+    sl = R.alibi_slopes(4)
+    pm = (np.arange(512)[None, :] < np.array([[100], [300]])).astype(np.int32)
+    docs = (np.arange(6144)[None, :] >= 2900).astype(np.int32)
+    return {
+        "no_bias_cross": dict(B=2, Sq=128, Sk=64, H=4, D=64, n=8),
+        "no_bias_ragged_shards": dict(B=1, Sq=600, Sk=408, H=2, D=128, n=3),
+        "causal_c1": dict(B=1, Sq=1024, Sk=1024, H=4, D=64, n=4, fn=ra.causal_bias(), ofn=R.make_bias_fn(causal=True)),
+        "causal_d128_ring8": dict(B=2, Sq=2048, Sk=2048, H=4, D=128, n=8, fn=ra.causal_bias(),
+                                  ofn=R.make_bias_fn(causal=True)),
+        "causal_long_shards": dict(B=1, Sq=6144, Sk=6144, H=2, D=128, n=3, fn=ra.causal_bias(),
+                                   ofn=R.make_bias_fn(causal=True)),
+        "more_steps_than_one_launch_takes": dict(B=1, Sq=2560, Sk=2560, H=2, D=64, n=20),
+        "window": dict(B=1, Sq=2048, Sk=2048, H=2, D=128, n=8, fn=ra.sliding_window_bias(300),
+                       ofn=R.make_bias_fn(causal=True, window=300), std=0.5),
+        "window_two_sided": dict(B=1, Sq=2048, Sk=2048, H=2, D=64, n=8, fn=ra.sliding_window_bias(200, causal=False),
+                                 ofn=R.make_bias_fn(window=200), std=0.5),
+        "segments_sorted": dict(B=2, Sq=2048, Sk=2048, H=2, D=128, n=4, fn=ra.segment_bias(),
+                                ofn=R.make_bias_fn(use_segments=True), qkw={"q_segment_ids": seg},
+                                kvkw={"kv_segment_ids": seg}),
+        "segments_random_causal": dict(B=2, Sq=512, Sk=512, H=4, D=64, n=8, fn=ra.causal_bias() + ra.segment_bias(),
+                                       ofn=R.make_bias_fn(causal=True, use_segments=True),
+                                       qkw={"q_segment_ids": segr}, kvkw={"kv_segment_ids": segr}),
+        "long_documents_causal": dict(B=1, Sq=6144, Sk=6144, H=2, D=128, n=2, std=0.7, fn=ra.causal_bias() + ra.segment_bias(),
+                                      ofn=R.make_bias_fn(causal=True, use_segments=True),
+                                      qkw={"q_segment_ids": docs}, kvkw={"kv_segment_ids": docs}),
+        "alibi_segments": dict(B=1, Sq=2048, Sk=2048, H=4, D=128, n=4, fn=ra.segment_bias() + ra.alibi_bias(sl),
+                               ofn=R.make_bias_fn(use_segments=True, alibi=sl), qkw={"q_segment_ids": seg[:1]},
+                               kvkw={"kv_segment_ids": seg[:1]}),
+        "prefix_lm": dict(B=2, Sq=512, Sk=512, H=2, D=64, n=4, fn=ra.prefix_lm_bias(),
+                          ofn=R.make_bias_fn(use_prefix=True), qkw={"q_prefix_mask": pm}, kvkw={"kv_prefix_mask": pm}),
+    }
+
+
+@pytest.mark.parametrize("name", sorted(_fused_cases()))
+def test_fused_ring_pass(device, name):
+    """block_impl="hip_fused": one launch per ring pass, the kernels walk the shards themselves.
+    Same oracle, same tolerances as the launch-per-step path."""
+    _check(device, "fused " + name, impl="hip_fused", **_fused_cases()[name])
+
+
+def test_fused_ring_pass_with_a_callable_bias_fn(device):
+    B, S, H, D, n = 2, 960, 2, 128, 3
+    q, k, v, do = R.make_inputs(7, B, S, S, H, D)
+    pos = np.broadcast_to(np.arange(S), (B, S))
+
+    def torch_fn(q_pos, kv_pos):
+        rel = q_pos[:, None, :, None] - kv_pos[:, None, None, :]
+        return torch.where(rel >= 0, -0.01 * rel.float(), -torch.inf)
+
+    bias = np.where(pos[:, None, :, None] >= pos[:, None, None, :],
+                    -0.01 * (pos[:, None, :, None] - pos[:, None, None, :]).astype(np.float32), -np.inf)
+    tq, tk, tv = (_dev(x, device, torch.bfloat16).requires_grad_(True) for x in (q, k, v))
+    tpos = _dev(pos, device)
+    out, lse = ra.ring_attention_with_lse(tq, tk, tv, n, bias_fn=torch_fn, bias_q_kwargs={"q_pos": tpos},
+                                          bias_kv_kwargs={"kv_pos": tpos}, out_dtype=torch.float32,
+                                          block_impl="hip_fused")
+    out.backward(_dev(do, device, torch.float32))
+    torch.cuda.synchronize()
+    want, want_lse = R.mha_dense(q, k, v, bias)
+    assert np.abs(out.detach().cpu().numpy() - want).max() <= OUT_TOL
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_TOL
+    for t, ref, nm in zip((tq, tk, tv), R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
+        mx, fro = _rel(t.grad.float().cpu().numpy(), ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+
+
+def test_multi_step_entry_points_equal_consecutive_steps(device):
+    """ra_fwd_steps / ra_bwd_dq_steps / ra_bwd_dkdv_steps against the same steps issued one by one
+    through ra_fwd_step / ra_bwd_step: the same sums in another rounding order."""
+    B, H, D, n, L = 1, 3, 128, 4, 640
+    S = n * L
+    q, k, v, do = R.make_inputs(11, B, S, S, H, D)
+    tq, tk, tv, tdo = (_dev(x, device, torch.bfloat16) for x in (q, k, v, do))
+    fn = ra.causal_bias()
+    sc = 1 / math.sqrt(D)
+    sh = lambda x, s: rr._shard_bhld(x, s, L)
+    bias = lambda qs, ks: rr.BlockBias(fn, qs * L, ks * L)
+    r = 2
+    order = [(r - t) % n for t in range(n)]  # the last one is fully masked
+    o1, m1, l1 = rr.init_carry(B, H, L, D, device)
+    for s in order:
+        rr.fwd_block(sh(tq, r), sh(tk, s), sh(tv, s), bias(r, s), o1, m1, l1, sc)
+    o2, m2, l2 = rr.init_carry(B, H, L, D, device)
+    rr.fwd_blocks(sh(tq, r), [(sh(tk, s), sh(tv, s)) for s in order], [bias(r, s) for s in order], o2, m2, l2, sc)
+    assert torch.equal(m1, m2)
+    torch.testing.assert_close(l2, l1, rtol=2e-3, atol=0)
+    torch.testing.assert_close(o2 / l2[..., None], o1 / l1[..., None], rtol=0, atol=4e-3)
+    lse = (m1 + l1.log()).contiguous()
+    out = (o1 / l1[..., None]).to(torch.bfloat16)
+    delta = rr.precompute_delta(out, sh(tdo, r))
+    z = lambda: torch.zeros((B, H, L, D), dtype=torch.float32, device=device)
+    dq1, dq2, dk_, dv_ = z(), z(), z(), z()
+    for s in order:
+        rr._bwd_step(sh(tq, r), sh(tk, s), sh(tv, s), sh(tdo, r), lse, delta, dq1, dk_, dv_, bias(r, s), sc, parts=2)
+    rr._bwd_steps("dq", [(sh(tq, r), sh(tk, s), sh(tv, s), sh(tdo, r), lse, delta, dq2, dk_, dv_, bias(r, s))
+                         for s in order], sc)
+    assert float(dk_.abs().max()) == 0.0 and float(dv_.abs().max()) == 0.0  # dq launches leave dk, dv alone
+    torch.testing.assert_close(dq2, dq1, rtol=0, atol=5e-3 * float(dq1.abs().max()))
+    # one key/value shard against all query shards (statistics of a plausible forward pass)
+    ks = 1
+    lse_all = torch.stack([lse + 0.1 * i for i in range(n)])
+    dl_all = torch.stack([delta * (1 + 0.1 * i) for i in range(n)])
+    dk1, dv1, dk2, dv2, dqx = z(), z(), z(), z(), z()
+    for qs in range(n):
+        rr._bwd_step(sh(tq, qs), sh(tk, ks), sh(tv, ks), sh(tdo, qs), lse_all[qs], dl_all[qs], dqx, dk1, dv1,
+                     bias(qs, ks), sc, parts=1)
+    rr._bwd_steps("dkdv", [(sh(tq, qs), sh(tk, ks), sh(tv, ks), sh(tdo, qs), lse_all[qs], dl_all[qs], dqx, dk2, dv2,
+                            bias(qs, ks)) for qs in range(n)], sc)
+    torch.cuda.synchronize()
+    assert float(dqx.abs().max()) == 0.0
+    torch.testing.assert_close(dk2, dk1, rtol=0, atol=5e-3 * float(dk1.abs().max()))
+    torch.testing.assert_close(dv2, dv1, rtol=0, atol=5e-3 * float(dv1.abs().max()))
+
+
 def test_delta_kernel(device):
     B, H, L, D = 2, 3, 100, 64
     rng = np.random.default_rng(0)
@@ -439,7 +559,8 @@ def test_fp32_and_fp16_inputs_are_cast(device):
 
 
 # ---- benchmark configs at full size -------------------------------------------------------------------------
-def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, bias_col, qkw=None, kvkw=None):
+def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, bias_col, qkw=None, kvkw=None,
+                   impl="hip"):
     """Full-size run on the GPU; the oracle is evaluated densely (fp64) on sampled query rows
     (out, lse, dq) and sampled key columns (dk, dv; these use the GPU's lse/out for the other
     rows, which the row samples vouch for), plus two exact invariants of softmax attention."""
@@ -449,7 +570,7 @@ def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, b
     q, k, v, do = mk(std), mk(std), mk(std), mk(1.0)
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
     out, lse = ra.ring_attention_with_lse(q, k, v, n, bias_fn=fn, bias_q_kwargs=qkw, bias_kv_kwargs=kvkw,
-                                          out_dtype=torch.float32)
+                                          out_dtype=torch.float32, block_impl=impl)
     out.backward(do.float())
     torch.cuda.synchronize()
     scale = 1 / math.sqrt(D)
@@ -503,6 +624,17 @@ def test_config2_full_size(device):
     cols = [0, 1023, 1024, 6000, S - 1]
     _sampled_check(device, "C2", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
                    lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf))
+
+
+def test_config2_full_size_fused(device):
+    # the same workload with one launch per ring pass: small shards are where that pays
+    B, H, D, S, n = 2, 16, 128, 8192, 8
+    pos = np.arange(S)
+    rows = [0, 1, 1023, 1024, 4095, 4096, 5000, S - 1]
+    cols = [0, 1023, 1024, 6000, S - 1]
+    _sampled_check(device, "C2 fused", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
+                   lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf),
+                   impl="hip_fused")
 
 
 def test_config3_full_size(device):
