@@ -153,6 +153,9 @@ def main():
     ap.add_argument("--impl", default="hip", choices=["hip", "hip_fused"],
                     help="hip: one launch per ring step (the headline); hip_fused: one launch per ring pass, "
                          "the kernels walk the shards themselves (no per-kernel roofline in that mode)")
+    ap.add_argument("--graph", action="store_true",
+                    help="capture one fwd+bwd pass of the ring in a HIP graph and time its replays (pays where "
+                         "launches are short: C2); no per-kernel roofline in that mode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
@@ -248,15 +251,41 @@ def main():
     for _ in range(args.warmup):
         one_step()
     torch.cuda.synchronize()
-    marks = [[ev(), ev(), ev()] for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        one_step(marks[i])
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt * 1e3 / args.steps
-    fwd_ms = sum(m[0].elapsed_time(m[1]) for m in marks) / args.steps
-    bwd_ms = sum(m[1].elapsed_time(m[2]) for m in marks) / args.steps
+    if args.graph:
+        args.no_kernel_timing = True
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            one_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            held = one_step()
+        graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ms_per_step = dt * 1e3 / args.steps
+        # the split is that of one eager pass (events cannot sit inside a replayed graph)
+        m = [ev(), ev(), ev()]
+        one_step(m)
+        torch.cuda.synchronize()
+        share = m[0].elapsed_time(m[1]) / m[0].elapsed_time(m[2])
+        fwd_ms, bwd_ms = ms_per_step * share, ms_per_step * (1.0 - share)
+    else:
+        marks = [[ev(), ev(), ev()] for _ in range(args.steps)]
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            one_step(marks[i])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        ms_per_step = dt * 1e3 / args.steps
+        fwd_ms = sum(m[0].elapsed_time(m[1]) for m in marks) / args.steps
+        bwd_ms = sum(m[1].elapsed_time(m[2]) for m in marks) / args.steps
     value = (flops_fwd + flops_bwd) / (ms_per_step * 1e-3) / 1e12
 
     result = {
@@ -266,7 +295,8 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}", "B": B, "H": H, "D": D, "S": S,
                    "ring_size": n, "bias": w["bias"], "unmasked_pairs_per_head": P,
-                   "launches": "one per ring pass" if fused else "one per ring step"},
+                   "launches": ("one per ring pass" if fused else "one per ring step") +
+                               (", replayed from a captured HIP graph" if args.graph else "")},
         "pct_of_bf16_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
         "fwd": {"ms": round(fwd_ms, 3), "tflops": round(flops_fwd / fwd_ms / 1e9, 2),
                 "pct_of_bf16_peak": round(100.0 * flops_fwd / fwd_ms / 1e9 / PEAK_BF16_TFLOPS, 2)},

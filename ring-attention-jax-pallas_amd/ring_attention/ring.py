@@ -340,6 +340,23 @@ class _RingPlan:
                 "consecutive inside every shard and identical across the batch")
         return [int(x) for x in starts[0].tolist()]
 
+    def live_steps(self, qs: Optional[int], ks: Optional[int]) -> int:
+        """How many ring steps of query shard ``qs`` (or key/value shard ``ks``) are not masked
+        entirely by the positional terms - the steps that cost something."""
+        fn = self.fn
+        if fn is None or not (fn.causal or fn.window):
+            return self.n
+        cnt = 0
+        for other in range(self.n):
+            q_lo = self.q_off[qs if qs is not None else other]
+            k_lo = self.kv_off[ks if ks is not None else other]
+            q_hi, k_hi = q_lo + self.Lq - 1, k_lo + self.Lk - 1
+            dead = fn.causal and k_lo > q_hi
+            if fn.window:
+                dead = dead or q_lo - k_hi >= fn.window or (not fn.causal and k_lo - q_hi >= fn.window)
+            cnt += not dead
+        return cnt
+
     def block_bias(self, qs: int, ks: int) -> Optional[BlockBias]:
         """Bias of (query shard qs, key/value shard ks)."""
         sl_q = slice(qs * self.Lq, (qs + 1) * self.Lq)
@@ -407,55 +424,102 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
     return out, lse
 
 
+_LANES = 2
+_lane_streams = {}
+
+
+def _run_in_lanes(jobs, costs):
+    """The ring passes of different shards do not depend on each other: spread them over
+    ``_LANES`` side streams (longest first, each to the lane with the least work so far) so that
+    launches too small to fill the GPU overlap.  ``jobs[j](lane)`` issues pass j on the current
+    stream using lane-private scratch ``lane``.  The caller's stream waits for all of them."""
+    main = torch.cuda.current_stream()
+    dev = main.device
+    if dev not in _lane_streams:
+        _lane_streams[dev] = [torch.cuda.Stream(device=dev) for _ in range(_LANES)]
+    lanes = _lane_streams[dev]
+    for st in lanes:
+        st.wait_stream(main)
+    load = [0.0] * _LANES
+    for j in sorted(range(len(jobs)), key=lambda j: -costs[j]):
+        i = load.index(min(load))
+        load[i] += costs[j]
+        with torch.cuda.stream(lanes[i]):
+            jobs[j](i)
+    for st in lanes:
+        main.wait_stream(st)
+
+
 def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO_TIMER):
     """``_ring_forward`` with the whole ring pass of a query shard in one launch: the kernel
-    visits the key/value shards in ring order itself."""
+    visits the key/value shards in ring order itself.  The passes of the emulated devices run
+    on two streams."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
     lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    o, m, l = init_carry(B, H, Lq, D, dev)
-    for r in range(n):
-        if r:
-            reset_carry(o, m, l)
-        order = [(r - t) % n for t in range(n)]  # ring.py:51-55
-        with timer.span("fwd_pass", r, -1):
-            fwd_blocks(_shard_bhld(q, r, Lq), [(_shard_bhld(k, s, Lk), _shard_bhld(v, s, Lk)) for s in order],
-                       [plan.block_bias(r, s) for s in order], o, m, l, sm_scale)
-        finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
+    carry = [init_carry(B, H, Lq, D, dev) for _ in range(_LANES)]
+    fresh = [True] * _LANES
+
+    def job(r):
+        def run(lane):
+            o, m, l = carry[lane]
+            if not fresh[lane]:
+                reset_carry(o, m, l)
+            fresh[lane] = False
+            order = [(r - t) % n for t in range(n)]  # ring.py:51-55
+            with timer.span("fwd_pass", r, -1):
+                fwd_blocks(_shard_bhld(q, r, Lq), [(_shard_bhld(k, s, Lk), _shard_bhld(v, s, Lk)) for s in order],
+                           [plan.block_bias(r, s) for s in order], o, m, l, sm_scale)
+            finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
+        return run
+
+    _run_in_lanes([job(r) for r in range(n)], [plan.live_steps(r, None) for r in range(n)])
     return out, lse
 
 
 def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
     """``_ring_backward`` with one launch per key/value shard for dK / dV (the kernel visits the
-    query shards in the order they arrive, ring.py:195) and one per query shard for dQ."""
+    query shards in the order they arrive, ring.py:195) and one per query shard for dQ; the
+    launches are independent of each other and run on two streams."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
     for s in range(n):
         precompute_delta(_shard_bhld(out, s, Lq), _shard_bhld(do, s, Lq), delta[s])
     dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
-    dk_acc = torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)
-    dv_acc = torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)
+    dkv_acc = [(torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev),
+                torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)) for _ in range(_LANES)]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
-    def step(qs, ks):
+    def step(qs, ks, dk_acc, dv_acc):
         return (_shard_bhld(q, qs, Lq), _shard_bhld(k, ks, Lk), _shard_bhld(v, ks, Lk),
                 _shard_bhld(do, qs, Lq), lse[qs], delta[qs], dq_acc[qs], dk_acc, dv_acc,
                 plan.block_bias(qs, ks))
 
-    for r in range(n):
-        dk_acc.zero_()
-        dv_acc.zero_()
-        with timer.span("bwd_dkdv_pass", -1, r):
-            _bwd_steps("dkdv", [step((r - t) % n, r) for t in range(n)], sm_scale)
-        _finalize_grad(dk_acc, _shard_bhld(dk, r, Lk))
-        _finalize_grad(dv_acc, _shard_bhld(dv, r, Lk))
-    for s in range(n):
-        # query shard s meets key/value shard r at step (r - s) mod n of device r
-        with timer.span("bwd_dq_pass", s, -1):
-            _bwd_steps("dq", [step(s, (s + t) % n) for t in range(n)], sm_scale)
-        _finalize_grad(dq_acc[s], _shard_bhld(dq, s, Lq))
+    def dkdv_job(r):
+        def run(lane):
+            dk_acc, dv_acc = dkv_acc[lane]
+            dk_acc.zero_()
+            dv_acc.zero_()
+            with timer.span("bwd_dkdv_pass", -1, r):
+                _bwd_steps("dkdv", [step((r - t) % n, r, dk_acc, dv_acc) for t in range(n)], sm_scale)
+            _finalize_grad(dk_acc, _shard_bhld(dk, r, Lk))
+            _finalize_grad(dv_acc, _shard_bhld(dv, r, Lk))
+        return run
+
+    def dq_job(s):
+        def run(lane):
+            dk_acc, dv_acc = dkv_acc[lane]  # not touched by a dQ launch
+            # query shard s meets key/value shard r at step (r - s) mod n of device r
+            with timer.span("bwd_dq_pass", s, -1):
+                _bwd_steps("dq", [step(s, (s + t) % n, dk_acc, dv_acc) for t in range(n)], sm_scale)
+            _finalize_grad(dq_acc[s], _shard_bhld(dq, s, Lq))
+        return run
+
+    jobs = [dkdv_job(r) for r in range(n)] + [dq_job(s) for s in range(n)]
+    costs = [8.0 * plan.live_steps(None, r) for r in range(n)] + [6.0 * plan.live_steps(s, None) for s in range(n)]
+    _run_in_lanes(jobs, costs)
     return dq, dk, dv
 
 

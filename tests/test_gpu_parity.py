@@ -516,6 +516,50 @@ def test_multi_step_entry_points_equal_consecutive_steps(device):
     torch.testing.assert_close(dv2, dv1, rtol=0, atol=5e-3 * float(dv1.abs().max()))
 
 
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_ring_replays_from_a_captured_graph(device, impl):
+    """Every launch of a forward + backward ring goes to the caller's stream (and, for the fused
+    passes, to side streams forked from it and joined back), allocates through torch only and
+    clears memory with fill kernels: the whole of it can be captured in a HIP graph.  Replays,
+    with eager work and synchronisations between them, reproduce the eager result bit for bit."""
+    B, S, H, D, n = 1, 2048, 4, 128, 4
+    q, k, v, do = (_dev(x, device, torch.bfloat16) for x in R.make_inputs(3, B, S, S, H, D))
+    seg = _dev(R.geometric_segment_ids(1, B, S, 500), device)
+    plan = rr._RingPlan(q, k, n, ra.causal_bias() + ra.segment_bias(), {"q_segment_ids": seg},
+                        {"kv_segment_ids": seg})
+    sc = 1 / math.sqrt(D)
+    fwd = rr._ring_forward_fused if impl == "hip_fused" else rr._ring_forward
+    bwd = rr._ring_backward_fused if impl == "hip_fused" else rr._ring_backward
+
+    def step():
+        out, lse = fwd(q, k, v, plan, sc, torch.bfloat16)
+        return (out, lse) + tuple(bwd(q, k, v, out, lse, do, plan, sc))
+
+    eager = [t.clone() for t in step()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm-up off the default stream, as capture requires
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    torch.cuda.synchronize()
+    for _ in range(3):
+        for t in captured:
+            t.fill_(0) if t.dtype != torch.bfloat16 else t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want)
+        again = step()  # eager work between the replays
+        torch.cuda.synchronize()
+        for got, want in zip(again, eager):
+            assert torch.equal(got, want)
+
+
 def test_delta_kernel(device):
     B, H, L, D = 2, 3, 100, 64
     rng = np.random.default_rng(0)

@@ -85,6 +85,28 @@ def test_ring_plan_shards_and_offsets():
         rr._RingPlan(q, k, 4, None, {"q_segment_ids": seg_q}, {})
 
 
+def test_ring_plan_counts_the_steps_that_cost_something():
+    q = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16)
+    plan = rr._RingPlan(q, q, 4, ra.causal_bias(), None, None)
+    assert [plan.live_steps(r, None) for r in range(4)] == [1, 2, 3, 4]
+    assert [plan.live_steps(None, r) for r in range(4)] == [4, 3, 2, 1]
+    plan = rr._RingPlan(q, q, 4, ra.sliding_window_bias(18), None, None)  # shards of 16 tokens
+    assert [plan.live_steps(r, None) for r in range(4)] == [1, 2, 3, 3]
+    plan = rr._RingPlan(q, q, 4, ra.sliding_window_bias(5, causal=False), None, None)
+    assert [plan.live_steps(r, None) for r in range(4)] == [2, 3, 3, 2]
+    assert rr._RingPlan(q, q, 4, None, None, None).live_steps(2, None) == 4
+    # agrees with the library's own classification of a step
+    lib = rr._lib.load()
+    for fn in (ra.causal_bias(), ra.sliding_window_bias(17), ra.sliding_window_bias(18), ra.sliding_window_bias(5, causal=False)):
+        plan = rr._RingPlan(q, q, 4, fn, None, None)
+        for r in range(4):
+            live = 0
+            for s in range(4):
+                st = plan.block_bias(r, s).to_struct(torch.device("cpu"))
+                live += not lib.ra_step_is_skippable(st, 16, 16)
+            assert plan.live_steps(r, None) == live
+
+
 def test_ring_plan_with_a_callable_bias_fn():
     # the reference's general form: the callable sees the shards of its kwargs (ring.py:107,186)
     q = torch.zeros(2, 64, 2, 64, dtype=torch.bfloat16)
