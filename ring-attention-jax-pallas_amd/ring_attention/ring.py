@@ -424,23 +424,37 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
     return out, lse
 
 
-_LANES = 2
+_MAX_LANES = 2
 _lane_streams = {}
 
 
-def _run_in_lanes(jobs, costs):
+def _lane_count(plan: "_RingPlan", device) -> int:
+    """Two lanes while one pass leaves compute units idle (its forward / dQ grid, one workgroup of
+    256 query rows per compute unit at a time, is smaller than two rounds of the chip); passes
+    that fill the GPU on their own run faster one after the other (measured: 8 shards of 1024
+    tokens gain a third from the second stream, 8 shards of 16384 lose 2 %)."""
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    workgroups = plan.B * plan.H * ((plan.Lq + 255) // 256)
+    return _MAX_LANES if workgroups < 2 * cus else 1
+
+
+def _run_in_lanes(jobs, costs, n_lanes):
     """The ring passes of different shards do not depend on each other: spread them over
-    ``_LANES`` side streams (longest first, each to the lane with the least work so far) so that
+    ``n_lanes`` side streams (longest first, each to the lane with the least work so far) so that
     launches too small to fill the GPU overlap.  ``jobs[j](lane)`` issues pass j on the current
     stream using lane-private scratch ``lane``.  The caller's stream waits for all of them."""
+    if n_lanes == 1:
+        for job in jobs:
+            job(0)
+        return
     main = torch.cuda.current_stream()
     dev = main.device
     if dev not in _lane_streams:
-        _lane_streams[dev] = [torch.cuda.Stream(device=dev) for _ in range(_LANES)]
-    lanes = _lane_streams[dev]
+        _lane_streams[dev] = [torch.cuda.Stream(device=dev) for _ in range(_MAX_LANES)]
+    lanes = _lane_streams[dev][:n_lanes]
     for st in lanes:
         st.wait_stream(main)
-    load = [0.0] * _LANES
+    load = [0.0] * n_lanes
     for j in sorted(range(len(jobs)), key=lambda j: -costs[j]):
         i = load.index(min(load))
         load[i] += costs[j]
@@ -452,14 +466,15 @@ def _run_in_lanes(jobs, costs):
 
 def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO_TIMER):
     """``_ring_forward`` with the whole ring pass of a query shard in one launch: the kernel
-    visits the key/value shards in ring order itself.  The passes of the emulated devices run
-    on two streams."""
+    visits the key/value shards in ring order itself.  Passes too small to fill the GPU run
+    on two streams (``_lane_count``)."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
     lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    carry = [init_carry(B, H, Lq, D, dev) for _ in range(_LANES)]
-    fresh = [True] * _LANES
+    n_lanes = _lane_count(plan, dev)
+    carry = [init_carry(B, H, Lq, D, dev) for _ in range(n_lanes)]
+    fresh = [True] * n_lanes
 
     def job(r):
         def run(lane):
@@ -474,22 +489,23 @@ def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO
             finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
         return run
 
-    _run_in_lanes([job(r) for r in range(n)], [plan.live_steps(r, None) for r in range(n)])
+    _run_in_lanes([job(r) for r in range(n)], [plan.live_steps(r, None) for r in range(n)], n_lanes)
     return out, lse
 
 
 def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
     """``_ring_backward`` with one launch per key/value shard for dK / dV (the kernel visits the
     query shards in the order they arrive, ring.py:195) and one per query shard for dQ; the
-    launches are independent of each other and run on two streams."""
+    launches are independent of each other and, when small, run on two streams."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
     for s in range(n):
         precompute_delta(_shard_bhld(out, s, Lq), _shard_bhld(do, s, Lq), delta[s])
     dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
+    n_lanes = _lane_count(plan, dev)
     dkv_acc = [(torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev),
-                torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)) for _ in range(_LANES)]
+                torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)) for _ in range(n_lanes)]
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
     def step(qs, ks, dk_acc, dv_acc):
@@ -519,7 +535,7 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
 
     jobs = [dkdv_job(r) for r in range(n)] + [dq_job(s) for s in range(n)]
     costs = [8.0 * plan.live_steps(None, r) for r in range(n)] + [6.0 * plan.live_steps(s, None) for s in range(n)]
-    _run_in_lanes(jobs, costs)
+    _run_in_lanes(jobs, costs, n_lanes)
     return dq, dk, dv
 
 

@@ -442,6 +442,13 @@ def test_fused_ring_pass(device, name):
     _check(device, "fused " + name, impl="hip_fused", **_fused_cases()[name])
 
 
+def test_fused_ring_pass_on_one_stream(device, monkeypatch):
+    # passes that fill the GPU on their own are issued one after the other on the caller's stream
+    monkeypatch.setattr(rr, "_MAX_LANES", 1)
+    _check(device, "fused, one stream", impl="hip_fused", **_fused_cases()["causal_d128_ring8"])
+    _check(device, "fused, one stream", impl="hip_fused", **_fused_cases()["segments_sorted"])
+
+
 def test_fused_ring_pass_with_a_callable_bias_fn(device):
     B, S, H, D, n = 2, 960, 2, 128, 3
     q, k, v, do = R.make_inputs(7, B, S, S, H, D)
