@@ -567,6 +567,52 @@ def test_ring_replays_from_a_captured_graph(device, impl):
             assert torch.equal(got, want)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_configurations(device, seed):
+    """Seeded random shapes (ragged shard lengths, cross attention, padded head dims, ring sizes
+    1..8) and bias combinations, each through both launch schemes, against the dense oracle."""
+    rng = np.random.default_rng(seed)
+    for case in range(12):
+        B, H = int(rng.integers(1, 3)), int(rng.choice([1, 2, 4]))
+        D = int(rng.choice([64, 128, 32, 96]))
+        n = int(rng.choice([1, 2, 3, 4, 8]))
+        Lq = int(rng.choice([3, 17, 64, 100, 128, 200, 256, 300, 520]))
+        cross = rng.random() < 0.3
+        Lk = int(rng.choice([5, 64, 96, 128, 250, 400])) if cross else Lq
+        Sq, Sk = n * Lq, n * Lk
+        kind = str(rng.choice(["none", "causal", "window", "window2", "seg", "seg_causal", "alibi",
+                               "alibi_causal_seg", "prefix"]))
+        if cross and kind == "prefix":
+            kind = "seg"
+        if rng.random() < 0.6:
+            segq = np.sort(rng.integers(0, max(2, Sq // 150), (B, Sq)).astype(np.int32), axis=1)
+        else:
+            segq = rng.integers(0, 3, (B, Sq)).astype(np.int32)
+        segk = segq if not cross else np.sort(rng.integers(0, max(2, Sq // 150), (B, Sk)).astype(np.int32), axis=1)
+        seg_kw = ({"q_segment_ids": segq}, {"kv_segment_ids": segk})
+        sl = R.alibi_slopes(H)
+        w = int(rng.integers(1, max(2, Sk)))
+        pm = (np.arange(Sq)[None] < rng.integers(0, Sq, (B, 1))).astype(np.int32)
+        fn, ofn, (qkw, kvkw) = {
+            "none": (None, None, ({}, {})),
+            "causal": (ra.causal_bias(), R.make_bias_fn(causal=True), ({}, {})),
+            "window": (ra.sliding_window_bias(w), R.make_bias_fn(causal=True, window=w), ({}, {})),
+            "window2": (ra.sliding_window_bias(w, causal=False), R.make_bias_fn(window=w), ({}, {})),
+            "seg": (ra.segment_bias(), R.make_bias_fn(use_segments=True), seg_kw),
+            "seg_causal": (ra.segment_bias() + ra.causal_bias(), R.make_bias_fn(causal=True, use_segments=True), seg_kw),
+            "alibi": (ra.alibi_bias(sl), R.make_bias_fn(alibi=sl), ({}, {})),
+            "alibi_causal_seg": (ra.alibi_bias(sl) + ra.causal_bias() + ra.segment_bias(),
+                                 R.make_bias_fn(causal=True, use_segments=True, alibi=sl), seg_kw),
+            "prefix": (ra.prefix_lm_bias(), R.make_bias_fn(use_prefix=True),
+                       ({"q_prefix_mask": pm}, {"kv_prefix_mask": pm})),
+        }[kind]
+        std = float(rng.choice([0.5, 1.0]))
+        data_seed = int(rng.integers(1 << 30))
+        for impl in ("hip", "hip_fused"):
+            _check(device, f"random {seed}.{case} {kind}", B, Sq, Sk, H, D, n, fn, ofn, qkw, kvkw, std=std,
+                   seed=data_seed, impl=impl)
+
+
 def test_delta_kernel(device):
     B, H, L, D = 2, 3, 100, 64
     rng = np.random.default_rng(0)
