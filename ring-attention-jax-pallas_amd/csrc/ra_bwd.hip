@@ -1015,7 +1015,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   constexpr int CPR = D / 8;   // 16-byte chunks per row
   constexpr int RPW = 4;       // rows per wave per tile
   // D = 128: one load instruction = 4 rows; D = 64: lanes 0..31 cover the wave's 4 rows
-  const bool ld_lane_on = (lane / CPR) < RPW;
+  // (with D = 128 every lane takes part, and the compiler need not mask anything)
+  const bool ld_lane_on = (64 / CPR <= RPW) || (lane / CPR) < RPW;
   const int ld_row = RPW * wave + (lane / CPR) % RPW;
   const int ld_chunk = ((tile_off<D>(ld_row, lane % CPR) - ld_row * ROWB) >> 4) * 8;
   const unsigned k_voff = (unsigned)(((long long)((lane / CPR) % RPW) * a.k.sl + ld_chunk) * 2);
@@ -1161,13 +1162,17 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
   int plain_lo = 0, plain_hi = 0;
+  // ordinal of tile t inside the run: t - run_tile0
+  int run_tile0 = j_lo;
+  if (run_hi > run_lo) {
+    int sbu;
+    run_tile0 = tile_at(run_lo, sbu) - run_lo;
+  }
+  run_tile0 = __builtin_amdgcn_readfirstlane(run_tile0);
   if (wave_on && lse_in_range && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
     key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
-    // ordinal of tile t inside the run: t - (first tile of the run) + run_lo
-    int sbu;
-    const int run_tile0 = (run_hi > run_lo) ? tile_at(run_lo, sbu) - run_lo : j_lo;
     plain_lo = max(lo - run_tile0, run_lo);
     plain_hi = max(min(hi - run_tile0, run_hi), plain_lo);
   }
@@ -1244,8 +1249,30 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     cur_valid = nxt_valid;
   };
 
+  // Loads of the plain stretch: consecutive complete tiles, so the wave-uniform global addresses
+  // advance by a constant and stay in scalar registers; nobody reads the ids of plain tiles.
+  const bf16_t* k_run = kbase;
+  const bf16_t* v_run = vbase;
+  auto seek_plain = [&](int tile) {
+    k_run = kbase + (long long)(tile * kDqKeyTile + RPW * wave_u) * a.k.sl;
+    v_run = vbase + (long long)(tile * kDqKeyTile + RPW * wave_u) * a.v.sl;
+  };
+  auto issue_run = [&](int buf) {
+    unsigned kvo = k_voff, vvo = v_voff;
+    if (TIGHT) {
+      kvo = s_voff[tid][0];
+      vvo = s_voff[tid][1];
+    }
+    if (ld_lane_on) {
+      global_to_lds16_s(k_run, kvo, RA_LDS_ADDR(&s_k[0][0]) + buf * TILE_BYTES + wave_u * RPW * ROWB);
+      global_to_lds16_s(v_run, vvo, RA_LDS_ADDR(&s_v[0][0]) + buf * TILE_BYTES + wave_u * RPW * ROWB);
+    }
+    k_run += (long long)kDqKeyTile * a.k.sl;
+    v_run += (long long)kDqKeyTile * a.v.sl;
+  };
+
   // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
-  // exists, so there is nothing to classify and no flag to consult.  Waves 4..7 take the
+  // exists and is complete, so there is nothing to classify and no flag to consult.  Waves 4..7 take the
   // iteration's barrier between the two MFMA blocks instead of before them (see below).
   const bool late_half = wave_u >= 4;
   auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
@@ -1280,10 +1307,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         fra[o2] = nat_frag((o2 & 1) ? vn : kn, o2 >> 1);
       }
       acc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frb[op], dsf[op / DB], acc[op % DB], 0, 0, 0);
-      if (op == 0) {  // next loads: their issue hides behind the MFMAs
-        int sbu;
-        issue_tile(tile_at(i + 3, sbu), PH3, false);  // plain tiles: nobody reads their ids
-      }
+      if (op == 0) issue_run(PH3);  // next loads: their issue hides behind the MFMAs
       __builtin_amdgcn_sched_barrier(0);
     }
     if (late_half) {
@@ -1365,7 +1389,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
   // iteration i is plain for plain_lo < i < plain_end
-  const int plain_end = __builtin_amdgcn_readfirstlane(DENSE ? -1 : min(plain_hi - 1, min(run_hi, n) - 3));
+  // (tile i+3 must exist, belong to the run and be complete)
+  const int plain_end = __builtin_amdgcn_readfirstlane(
+      DENSE ? -1 : min(min(plain_hi - 1, min(run_hi, n) - 3), a.Lk / kDqKeyTile - run_tile0 - 3));
   int i = 0;
   for (; i < n && !(i > plain_lo && i + 6 <= plain_end); i += 6) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
@@ -1377,6 +1403,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   }
   if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
     const bool stretch = i + 6 <= plain_end;
+    if (stretch) seek_plain(run_tile0 + i + 3);
     if (GENERAL && stretch) seg_r = pre_r = 0;  // stored already; not carried through the stretch
     if (stretch) {
       // the two row constants of the stretch replace the two of the generic iterations, which
