@@ -170,3 +170,18 @@ def test_multi_step_entry_points_validate_before_any_gpu_call(lib):
             p.bias.flags = _lib.RA_BIAS_CAUSAL
             p.bias.kv_offset = 1 << 20
         assert fn(arr, 2, None) == 0
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/ring_attention_hip.h must compile as C99 on its own (no HIP, no C++)."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "hdr.c"
+    src.write_text('#include "ring_attention_hip.h"\n'
+                   "int main(void) { ra_fwd_step_params p; (void)p; return RA_OK; }\n")
+    res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only",
+                          "-I", os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
