@@ -25,13 +25,91 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
 
-# HBM bytes per launch (read + written) of the step kernels, measured with
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script (`--copy-probe` gives the
-# 1 GiB copy the counters are scaled by: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Profiler counters
-# cannot be read from inside a timed run, so the figures are carried here.
-MEASURED_HBM_BYTES_PER_LAUNCH = {
-    "C3b": {"fwd_step_kernel": 1.492e9, "dkdv_kernel": 2.412e9, "dq_kernel": 1.429e9},
-}
+CSRC = os.path.join(ROOT, "ring-attention-jax-pallas_amd", "csrc")
+
+
+def csrc_digest():
+    """Digest of the kernel sources: a stored profiler figure is only quoted while it matches."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h")):
+            with open(os.path.join(CSRC, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+def stored_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 counter summary of this
+    workload (profiles/<workload>_hbm_traffic.txt, written by --pmc-summary).  Profiler counters
+    cannot be read from inside a timed run; the summary carries the digest of the kernel sources
+    it was measured on, and a figure measured on other sources is not quoted (None)."""
+    path = os.path.join(ROOT, "profiles", f"{workload.lower()}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    digest, table = None, {}
+    with open(path) as f:
+        for line in f:
+            t = line.split()
+            if line.startswith("csrc-digest:"):
+                digest = t[1]
+            elif len(t) == 3 and t[0] == "bytes-per-launch":
+                table[t[1]] = float(t[2])
+    if digest != csrc_digest():
+        return None
+    return table.get(kernel)
+
+
+def pmc_summary(workload, fetch_csv, write_csv):
+    """Text summary of two rocprofv3 --pmc runs of `bench.py --copy-probe` (FETCH_SIZE, WRITE_SIZE).
+    Both counters are scaled by what they read for the 1 GiB elementwise copy of --copy-probe."""
+    import csv
+    from collections import defaultdict
+
+    def read(path, counter):
+        tot, cnt = defaultdict(float), defaultdict(int)
+        with open(path) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] != counter:
+                    continue
+                tot[row["Kernel_Name"]] += float(row["Counter_Value"])
+                cnt[row["Kernel_Name"]] += 1
+        return {k: (tot[k] / cnt[k], cnt[k]) for k in tot}
+
+    fetch, write = read(fetch_csv, "FETCH_SIZE"), read(write_csv, "WRITE_SIZE")
+    # the copy probe: the kernel outside this library whose writes are closest to 1 GiB per launch
+    gib_kib = float(1 << 20)
+    probe = [k for k in fetch if "ra::" not in k and k in write]
+    pk = min(probe, key=lambda k: abs(write[k][0] - gib_kib), default=None)
+    if pk is None or abs(write[pk][0] - gib_kib) > 0.2 * gib_kib:
+        raise SystemExit("no copy-probe kernel in the counter files: run bench.py with --copy-probe")
+    f_scale = gib_kib / fetch[pk][0]
+    w_scale = gib_kib / write[pk][0]
+    out = [f"rocprofv3 HBM byte counters, workload {workload}: one fwd+bwd pass of the ring",
+           "commands (from /tmp, TMPDIR=/tmp, R = repository root), one counter per run:",
+           f"  rocprofv3 --pmc FETCH_SIZE --output-format csv -d $R/gpurun_out/pmc_fetch -o f -- python3 $R/bench.py --workload {workload} --steps 1 --warmup 0 --no-cpu-baseline --no-kernel-timing --copy-probe",
+           f"  rocprofv3 --pmc WRITE_SIZE --output-format csv -d $R/gpurun_out/pmc_write -o w -- python3 $R/bench.py --workload {workload} --steps 1 --warmup 0 --no-cpu-baseline --no-kernel-timing --copy-probe",
+           f"  python3 $R/bench.py --workload {workload} --pmc-summary <f_counter_collection.csv> <w_counter_collection.csv>",
+           f"calibration kernel (reads 1 GiB, writes 1 GiB): {pk[:60]}",
+           f"  FETCH_SIZE reads {fetch[pk][0]:.0f} KiB -> scale {f_scale:.3f};  WRITE_SIZE reads {write[pk][0]:.0f} KiB -> scale {w_scale:.3f}",
+           f"csrc-digest: {csrc_digest()}",
+           "", f"{'kernel':<44}{'n':>5}{'FETCH KiB':>14}{'WRITE KiB':>14}{'read GB':>10}{'written GB':>12}"]
+    rows = []
+    for k in sorted(fetch):
+        if not k.startswith("ra::") and "ra::" not in k:
+            continue
+        fa, n = fetch[k]
+        wa = write.get(k, (0.0, 0))[0]
+        rd, wr = fa * f_scale * 1024.0, wa * w_scale * 1024.0
+        short = k.split("(")[0].replace("void ", "")
+        out.append(f"{short:<44}{n:>5}{fa:>14.0f}{wa:>14.0f}{rd / 1e9:>10.3f}{wr / 1e9:>12.3f}")
+        rows.append((short, rd + wr))
+    out.append("")
+    out.append("HBM bytes per launch (read + written, scaled); bench.py quotes these as roofline.traffic:")
+    for short, tot in rows:
+        out.append(f"bytes-per-launch {short.replace('ra::', '').split('<')[0]} {tot:.4e}")
+    return "\n".join(out) + "\n"
+
 
 WORKLOADS = {
     # name: (B, H, D, S, ring, bias, std, description)
@@ -99,7 +177,12 @@ def mfma_ceiling(torch, dev):
     power management leaves of the published peak.  Reported next to `roofline`, never used in it."""
     import ctypes as C
     from ring_attention import _lib
-    lib = _lib.load()
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libringattn_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build the kernels first (__graft_entry__.build())")
+    lib = C.CDLL(path)
+    lib.ra_probe_mfma_rate.restype = C.c_int
+    lib.ra_probe_mfma_rate.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     iters = 100000
     sink = torch.empty(cus * 256, device=dev, dtype=torch.float32)
@@ -108,7 +191,9 @@ def mfma_ceiling(torch, dev):
     for rep in range(4):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record(torch.cuda.current_stream())
-        _lib.check("ra_probe_mfma_rate", lib.ra_probe_mfma_rate(sink.data_ptr(), cus, iters, 1, stream))
+        rc = lib.ra_probe_mfma_rate(sink.data_ptr(), cus, iters, 1, stream)
+        if rc:
+            raise RuntimeError(f"ra_probe_mfma_rate failed with code {rc}")
         b.record(torch.cuda.current_stream())
         torch.cuda.synchronize()
         if rep:  # the first launch runs while the clock is still ramping
@@ -117,9 +202,10 @@ def mfma_ceiling(torch, dev):
             "what": "v_mfma_f32_32x32x16_bf16 only, random operands in registers, one wave per SIMD, all CUs"}
 
 
-def cpu_baseline(D):
-    """The numpy restatement of the reference algorithm, timed on the host cores on a bounded
-    sample of the workload (same head dim, causal, fp32): H=8, S=16384 as 4 shards of 4096."""
+def cpu_baseline(D, config="sample"):
+    """The numpy restatement of the reference algorithm (fp32, causal) timed on the host cores:
+    a bounded sample with the workload's head dim (H=8, S=16384 as 4 shards of 4096), or
+    benchmark config C1 (forward only) or C2 (forward + backward) in full."""
     import numpy as np
     from oracle import ring_oracle as R
     try:
@@ -127,20 +213,30 @@ def cpu_baseline(D):
         threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
     except Exception:
         threads = os.cpu_count() or 1
-    H, S, n = 8, 16384, 4
-    q, k, v, do = R.make_inputs(0, 1, S, S, H, D)
-    pos = np.broadcast_to(np.arange(S), (1, S))
+    B, H, S, n, bwd = {"sample": (1, 8, 16384, 4, True), "C1": (1, 4, 1024, 4, False),
+                       "C2": (2, 16, 8192, 8, True)}[config]
+    if config == "C1":
+        D = 64
+    elif config == "C2":
+        D = 128
+    q, k, v, do = R.make_inputs(0, B, S, S, H, D)
+    pos = np.broadcast_to(np.arange(S), (B, S))
     fn = R.make_bias_fn(causal=True)
+    reps = 20 if config == "C1" else 1  # C1 takes milliseconds
     t0 = time.perf_counter()
-    out, lse = R.ring_attention(q, k, v, n, fn, {"q_positions": pos}, {"kv_positions": pos},
-                                dtype=np.float32, skip_masked_steps=True)
-    R.ring_attention_bwd(q, k, v, out, lse, do, n, fn, {"q_positions": pos}, {"kv_positions": pos},
-                         dtype=np.float32)
-    dt = time.perf_counter() - t0
-    flops = 14.0 * D * (S * (S + 1) / 2) * H
+    for _ in range(reps):
+        out, lse = R.ring_attention(q, k, v, n, fn, {"q_positions": pos}, {"kv_positions": pos},
+                                    dtype=np.float32, skip_masked_steps=True)
+        if bwd:
+            R.ring_attention_bwd(q, k, v, out, lse, do, n, fn, {"q_positions": pos}, {"kv_positions": pos},
+                                 dtype=np.float32)
+    dt = (time.perf_counter() - t0) / reps
+    flops = (14.0 if bwd else 4.0) * D * (S * (S + 1) / 2) * H * B
+    what = "fwd+bwd" if bwd else "fwd"
+    label = "a bounded sample" if config == "sample" else f"config {config} in full"
     return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
-            "sample": f"numpy fp32 restatement of ring_attention fwd+bwd, B=1 H={H} D={D} S={S} as {n} "
-                      f"shards, causal, {dt:.1f} s wall",
+            "sample": f"numpy fp32 restatement of ring_attention {what} on {label}: B={B} H={H} D={D} S={S} as "
+                      f"{n} shards, causal, {dt:.3g} s wall",
             "seconds": dt}
 
 
@@ -158,9 +254,19 @@ def main():
                          "launches are short: C2); no per-kernel roofline in that mode")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--cpu-baseline-config", default="sample", choices=["sample", "C1", "C2"],
+                    help="what the CPU restatement is timed on: a bounded sample with the workload's head dim "
+                         "(default, ~20 s), or benchmark config C1 / C2 in full")
+    ap.add_argument("--pmc-summary", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of this "
+                         "script (FETCH_SIZE, WRITE_SIZE; both with --copy-probe) into the text summary kept "
+                         "under profiles/ and print it")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain elementwise copy of 1 GiB (calibrates HBM byte counters)")
     args = ap.parse_args()
+    if args.pmc_summary:
+        sys.stdout.write(pmc_summary(args.workload, *args.pmc_summary))
+        return
     if args.gpus != 1:
         print("bench.py measures ONE GPU: the ring is emulated on a single MI355X and there is no "
               "multi-GPU path in this build (got --gpus %d)" % args.gpus, file=sys.stderr)
@@ -178,11 +284,23 @@ def main():
     w = WORKLOADS[args.workload]
     B, H, D, S, n = w["B"], w["H"], w["D"], w["S"], w["n"]
     L = S // n
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(0)
-    mk = lambda: (torch.randn((B, S, H, D), generator=gen, device=dev, dtype=torch.float32) * w["std"]).to(torch.bfloat16)
-    q, k, v = mk(), mk(), mk()
-    do = torch.randn((B, S, H, D), generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    # q, k, v ~ N(0, std^2), dO ~ N(0, 1) from numpy.random.default_rng(0) in fp32, rounded to bf16
+    # (round to nearest even) on the device: the same stream, draw for draw, as the oracle's
+    # make_inputs(0, B, S, S, H, D, std), generated in pieces to bound host memory
+    rng0 = np.random.default_rng(0)
+
+    def mk(std):
+        t = torch.empty(B * S * H * D, device=dev, dtype=torch.bfloat16)
+        piece = 1 << 26
+        for a0 in range(0, t.numel(), piece):
+            x = rng0.standard_normal(min(piece, t.numel() - a0), dtype=np.float32)
+            if std != 1.0:
+                x *= np.float32(std)
+            t[a0:a0 + x.size] = torch.from_numpy(x).to(dev).to(torch.bfloat16)
+        return t.view(B, S, H, D)
+
+    q, k, v = mk(w["std"]), mk(w["std"]), mk(w["std"])
+    do = mk(1.0)
     sm_scale = 1.0 / math.sqrt(D)
 
     q_kw = kv_kw = None
@@ -222,10 +340,11 @@ def main():
                 pairs[(qs, ks)] = pair_count(w["bias"], w.get("window", 0), qs * L, ks * L, L, L)
     only_rank = w.get("only_rank")
     if only_rank is not None:
-        # one device's real share: its query shard against all KV shards (forward), and the
-        # same (q, kv) pairs in the backward pass
-        raise SystemExit("C3a is measured through C3b's per-launch records; run --workload C3b")
-    P = sum(pairs.values())
+        # one device's real share: its query shard against all key/value shards in the forward
+        # pass and the same (query shard, key/value shard) pairs in the backward pass
+        P = sum(pairs[(only_rank, ks)] for ks in range(n))
+    else:
+        P = sum(pairs.values())
     flops_fwd = 4.0 * D * P * B * H
     flops_bwd = 10.0 * D * P * B * H
 
@@ -237,7 +356,48 @@ def main():
     if fused:
         args.no_kernel_timing = True
 
+    if only_rank is not None:
+        if fused or args.graph:
+            raise SystemExit("--workload C3a runs launch per step, eagerly")
+        args.no_kernel_timing = True
+        r = only_rank
+        qr, dor = rr._shard_bhld(q, r, L), rr._shard_bhld(do, r, L)
+        carry = rr.init_carry(B, H, L, D, dev)
+        out_r = torch.empty((B, L, H, D), dtype=torch.bfloat16, device=dev).permute(0, 2, 1, 3)
+        lse_r = torch.empty((B, H, L), dtype=torch.float32, device=dev)
+        delta_r = torch.empty((B, H, L), dtype=torch.float32, device=dev)
+        dq_acc = torch.empty((B, H, L, D), dtype=torch.float32, device=dev)
+        dk_acc, dv_acc = torch.empty_like(dq_acc), torch.empty_like(dq_acc)
+        dq_r = torch.empty((B, L, H, D), dtype=torch.bfloat16, device=dev).permute(0, 2, 1, 3)
+        dk, dv = torch.empty_like(k), torch.empty_like(v)
+        order = [(r - t) % n for t in range(n)]  # the key/value shards as they arrive at device r
+
+    def rank_step(marks=None):
+        if marks is not None:
+            marks[0].record()
+        rr.reset_carry(*carry)
+        for s_ in order:
+            rr.fwd_block(qr, rr._shard_bhld(k, s_, L), rr._shard_bhld(v, s_, L), plan.block_bias(r, s_), *carry, sm_scale)
+        rr.finalize_carry(*carry, out_r, lse_r)
+        if marks is not None:
+            marks[1].record()
+        rr.precompute_delta(out_r, dor, delta_r)
+        dq_acc.zero_()
+        for s_ in order:
+            dk_acc.zero_()
+            dv_acc.zero_()
+            rr._bwd_step(qr, rr._shard_bhld(k, s_, L), rr._shard_bhld(v, s_, L), dor, lse_r, delta_r, dq_acc,
+                         dk_acc, dv_acc, plan.block_bias(r, s_), sm_scale)
+            rr._finalize_grad(dk_acc, rr._shard_bhld(dk, s_, L))
+            rr._finalize_grad(dv_acc, rr._shard_bhld(dv, s_, L))
+        rr._finalize_grad(dq_acc, dq_r)
+        if marks is not None:
+            marks[2].record()
+        return out_r, (dq_r, dk, dv)
+
     def one_step(marks=None):
+        if only_rank is not None:
+            return rank_step(marks)
         if marks is not None:
             marks[0].record()
         out, lse = ring_fwd(q, k, v, plan, sm_scale, torch.bfloat16)
@@ -334,7 +494,7 @@ def main():
         result["roofline"] = {"bound": "mfma", "kernel": names[dom], "achieved": round(ach, 2),
                               "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                               "frac": round(ach / PEAK_BF16_TFLOPS, 4),
-                              "traffic": MEASURED_HBM_BYTES_PER_LAUNCH.get(args.workload, {}).get(names[dom])}
+                              "traffic": stored_traffic(args.workload, names[dom])}
         result["kernels"] = kernels
         # rank 7's share (the last query shard against all 8 KV shards)
         if args.workload == "C3b":
@@ -357,7 +517,7 @@ def main():
         del src, dst
 
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(D)
+        result["cpu_baseline"] = cpu_baseline(D, args.cpu_baseline_config)
     print(json.dumps(result))
 
 

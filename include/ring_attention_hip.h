@@ -22,6 +22,7 @@
  *    without a transpose;
  *  - carries and accumulators are fp32 and contiguous: o/dq/dk/dv [B, H, L, D],
  *    m/l/lse/delta [B, H, L];
+ *  - prefix masks are read as booleans: any non-zero value marks a prefix token;
  *  - D must be 64 or 128 and equal for q, k and v (the reference's kernels assume
  *    dk == dv too, ring_kernel.py:170,175); lengths may be any positive number.
  */
@@ -190,16 +191,6 @@ int ra_bwd_dkdv_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* st
  * identity on the carry and may be skipped; 0 otherwise.  The reference runs such steps and
  * lets its -inf guards nullify them (ring.py:66,69). */
 int ra_step_is_skippable(const ra_bias* bias, int32_t Lq, int32_t Lk);
-
-/* Diagnostic with no counterpart in the reference: launches `blocks` workgroups of four waves
- * (one per SIMD) that each issue iters x 8 independent v_mfma_f32_32x32x16_bf16 and nothing
- * else; the caller times the launch and divides blocks * 4 * iters * 8 * 32768 FLOP by it.  With
- * random_operands != 0 the operands toggle like real data.  `sink` receives blocks * 256 floats.
- * The rate obtained with one workgroup per compute unit is the ceiling that the board's power
- * management leaves to any kernel built from this instruction; bench.py reports it next to
- * the published peak. */
-int ra_probe_mfma_rate(float* sink, int32_t blocks, int32_t iters, int32_t random_operands,
-                       void* stream);
 
 /* Argument checks of ra_fwd_step / ra_bwd_step without launching anything (host only). */
 int ra_fwd_step_check(const ra_fwd_step_params* p);

@@ -42,6 +42,12 @@ int check_dims(int B, int H, int Lq, int Lk, int D) {
   if (Lq > kMaxLen || Lk > kMaxLen)
     return fail(RA_ERR_SHAPE, "shard length above %d tokens", kMaxLen);
   if ((int64_t)B * H > (1 << 20)) return fail(RA_ERR_SHAPE, "B*H too large");
+  // the smallest tile any kernel hands to a workgroup is 128 tokens: the flat grid of the launch
+  // must fit the 31 bits of a grid dimension
+  const int64_t tiles = ((int64_t)(Lq > Lk ? Lq : Lk) + 127) / 128;
+  if ((int64_t)B * H * tiles > 0x7fffffffll)
+    return fail(RA_ERR_SHAPE, "B*H*ceil(L/128) = %lld workgroups exceed the grid limit of 2^31-1",
+                (long long)((int64_t)B * H * tiles));
   if (D != 64 && D != 128) return fail(RA_ERR_HEAD_DIM, "head dim %d unsupported (64 or 128)", D);
   return RA_OK;
 }
@@ -171,7 +177,7 @@ void add_kv_shard(ra::KvShardList& sl, const ra_tensor& k, const ra_tensor& v, c
 
 extern "C" {
 
-int ra_version(void) { return 1002; }
+int ra_version(void) { return 1003; }
 
 const char* ra_last_error(void) { return g_err; }
 
@@ -308,6 +314,10 @@ int ra_fwd_finalize(const float* o, const float* m, const float* l, void* out, i
     return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
   if ((out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
     return fail(RA_ERR_ALIGN, "out strides must be multiples of 4 elements");
+  // the kernel stores four elements at a time: 8 bytes of bf16 or 16 bytes of fp32
+  if (reinterpret_cast<uintptr_t>(out) % (out_dtype == RA_DTYPE_F32 ? 16u : 8u))
+    return fail(RA_ERR_ALIGN, "out must be aligned to four elements (%d bytes)", out_dtype == RA_DTYPE_F32 ? 16 : 8);
+  if (!aligned16(o)) return fail(RA_ERR_ALIGN, "o is not 16-byte aligned");
   hipError_t e = ra::launch_fwd_finalize(o, m, l, out, out_dtype == RA_DTYPE_F32, out_stride_b,
                                          out_stride_h, out_stride_l, lse, B, H, Lq, D,
                                          (hipStream_t)stream);
@@ -433,17 +443,12 @@ int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t o
   if (rc) return rc;
   if ((out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
     return fail(RA_ERR_ALIGN, "out strides must be multiples of 4 elements");
+  // the kernel loads 16 bytes of fp32 and stores 8 bytes of bf16 at a time
+  if (reinterpret_cast<uintptr_t>(out) % 8u) return fail(RA_ERR_ALIGN, "out must be 8-byte aligned");
+  if (!aligned16(acc)) return fail(RA_ERR_ALIGN, "acc is not 16-byte aligned");
   hipError_t e = ra::launch_bwd_finalize(acc, out, out_stride_b, out_stride_h, out_stride_l, B, H, L,
                                          D, (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_finalize launch");
-}
-
-int ra_probe_mfma_rate(float* sink, int32_t blocks, int32_t iters, int32_t random_operands, void* stream) {
-  if (!sink) return fail(RA_ERR_NULL, "ra_probe_mfma_rate: sink is NULL");
-  if (blocks <= 0 || blocks > 65536 || iters <= 0 || (iters % 4))
-    return fail(RA_ERR_SHAPE, "ra_probe_mfma_rate: blocks in [1, 65536], iters a positive multiple of 4");
-  hipError_t e = ra::launch_mfma_rate(sink, blocks, iters, random_operands != 0, (hipStream_t)stream);
-  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_probe_mfma_rate launch");
 }
 
 }  // extern "C"

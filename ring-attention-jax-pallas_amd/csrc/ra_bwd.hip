@@ -14,20 +14,6 @@
 
 #include "ra_launch.h"
 
-#ifndef RA_ABLATE_B
-#define RA_ABLATE_B 0  // timing experiments only: bit mask of loop parts to leave out
-#endif
-
-#if defined(RA_PROFILE) && defined(PROF_DQ)
-#define RA_PROFQ_DECL RA_PROF_DECL
-#define RA_PROFQ_MARK(i, id) RA_PROF_MARK(i, id)
-#define RA_PROFQ_DUMP RA_PROF_DUMP
-#else
-#define RA_PROFQ_DECL
-#define RA_PROFQ_MARK(i, id) do { } while (0)
-#define RA_PROFQ_DUMP do { } while (0)
-#endif
-
 namespace ra {
 
 constexpr int kBwdMaxListTiles = 2048;
@@ -107,7 +93,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const int wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
-  RA_STAMP(0);
   const int nkt = (a.Lk + KEYS_WG - 1) / KEYS_WG;
   int hh, kt;
   decode_block(blockIdx.x, a.B * a.H, nkt, hh, kt);
@@ -176,8 +161,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(z8, z8, z16, 0, 0, 0);
     }
   }
-
-  RA_PROF_DECL
   // ---- one pass of everything below per query shard ------------------------------------------
   int q_off = bs.q_off;
   const bf16_t* q_ptr = a.q.ptr;
@@ -204,7 +187,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   }
   const int* q_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? q_seg_ptr + b * bs.q_seg_sb : nullptr;
   const int* q_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? q_pre_ptr + b * bs.q_pre_sb : nullptr;
-  RA_STAMP(1);
   // ---- which query tiles does this workgroup visit -------------------------------------------
   const int ntiles = (a.Lq + kQTile - 1) / kQTile;
   const int k_hi = min(k0 + KEYS_WG, a.Lk) - 1;
@@ -473,9 +455,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     if (n > 0) issue_tile(tile_at(0, sbu), 0, xr[0]);
     if (n > 1) issue_tile(tile_at(1, sbu), 1, xr[1]);
     if (n > 2) issue_tile(tile_at(2, sbu), 2, xr[2]);  // its statistics are stored in iteration 1
-    RA_STAMP(2);
     __builtin_amdgcn_s_waitcnt(0);
-    RA_STAMP(3);
     if (n > 0) store_stat(0, xr[0]);
     if (n > 1) store_stat(1, xr[1]);
   }
@@ -508,7 +488,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       if (needs_bias(qt0, segbit, cls)) prepare(s_a, qt0, segbit, cls, 0);
     }
   }
-  RA_STAMP(4);
   // P(i-1) and dS(i-1), packed in pairs, waiting for their dV / dK products
   u32x4 pfw[2], dsw[2];
 #pragma unroll
@@ -601,7 +580,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     const char* dop = s_do[PHP];
     const char* qn = s_q[PH1];
     const char* don = s_do[PH1];
-    RA_PROF_MARK(i, 1);
     // operands of the dV / dK products come from tile i-1, visible since two barriers ago
     bf16x8 frb[4 * DB];
 #pragma unroll
@@ -611,8 +589,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     // fetches above, and what other waves need (the statistics stored half an iteration ago) is
     // older than those.
     RA_WAIT_VMCNT(LPT);
-    if (!(RA_ABLATE_B & 4)) asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" : : "n"(2 * PFT) : "memory");
-    RA_PROF_MARK(i, 2);
+    asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" : : "n"(2 * PFT) : "memory");
     bf16x8 pf[2], dsf[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
@@ -636,21 +613,19 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       if (op & 1) dk[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dsf[ks], frb[op], dk[db], 0, 0, 0);
       else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], frb[op], dv[db], 0, 0, 0);
       // next tile's loads, one instruction group per MFMA: their issue hides behind the MFMAs
-      if (!(RA_ABLATE_B & 16)) {
-        if (op == 0) {
-          load_stat(st_run, xr[PH3 % 3]);
-          st_run += kQTile * 4;
-        }
-        if (op == 1) {
-          if (NLD == 2) global_to_lds16_s_x2(q_run, q_voff[0], q_run + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1], q_dst0 + PH3 * TILE_BYTES);
-          else global_to_lds16_s(q_run, q_voff[0], q_dst0 + PH3 * TILE_BYTES);
-          q_run += (long long)kQTile * a.q.sl;
-        }
-        if (op == 2) {
-          if (NLD == 2) global_to_lds16_s_x2(do_run, do_voff[0], do_run + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1], do_dst0 + PH3 * TILE_BYTES);
-          else global_to_lds16_s(do_run, do_voff[0], do_dst0 + PH3 * TILE_BYTES);
-          do_run += (long long)kQTile * a.dout.sl;
-        }
+      if (op == 0) {
+        load_stat(st_run, xr[PH3 % 3]);
+        st_run += kQTile * 4;
+      }
+      if (op == 1) {
+        if (NLD == 2) global_to_lds16_s_x2(q_run, q_voff[0], q_run + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1], q_dst0 + PH3 * TILE_BYTES);
+        else global_to_lds16_s(q_run, q_voff[0], q_dst0 + PH3 * TILE_BYTES);
+        q_run += (long long)kQTile * a.q.sl;
+      }
+      if (op == 2) {
+        if (NLD == 2) global_to_lds16_s_x2(do_run, do_voff[0], do_run + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1], do_dst0 + PH3 * TILE_BYTES);
+        else global_to_lds16_s(do_run, do_voff[0], do_dst0 + PH3 * TILE_BYTES);
+        do_run += (long long)kQTile * a.dout.sl;
       }
       // the statistics of tile i+1 are the initial values of S(i+1), dP(i+1)
       {
@@ -666,7 +641,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    RA_PROF_MARK(i, 3);
     // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA, the chain of
     // an element (exp2, product, packing) spread over consecutive slots
     float pe[16], de[16];
@@ -676,39 +650,34 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       if (op + PFN < 2 * KS) fra[op + PFN] = nat_frag(((op + PFN) & 1) ? don : qn, (op + PFN) >> 1);
       if (op & 1) mfma_scores(PN, fra[op], vfa[op >> 1]);
       else mfma_scores(SN, fra[op], kfa[op >> 1]);
-      if (op == 2 && !(RA_ABLATE_B & 32)) {
+      if (op == 2) {
         // the per-row word of tile i+2 is the oldest load but those of its tile and of tile i+3
         RA_WAIT_VMCNT(2 * LPT - 1);
         store_stat(PH2, xr[PH2 % 3]);
       }
-      if (!(RA_ABLATE_B & 8)) {
 #pragma unroll
-        for (int e = 0; e < EPO; ++e) {
-          const int r = op * EPO + e;
-          if (r < 16) {
-            pe[r] = fast_exp2(SC[r]);
-            asm volatile("" : "+v"(pe[r]));
-          }
-          if (r >= 1 && r <= 16) {
-            de[r - 1] = pe[r - 1] * PC[r - 1];
-            asm volatile("" : "+v"(de[r - 1]));
-          }
-          if (r >= 2 && r <= 16 && !(r & 1)) {
-            unsigned pw = pack2(pe[r - 2], pe[r - 1]), dw = pack2(de[r - 2], de[r - 1]);
-            asm volatile("" : "+v"(pw), "+v"(dw));
-            pfw[(r - 2) >> 3][((r - 2) & 7) >> 1] = pw;
-            dsw[(r - 2) >> 3][((r - 2) & 7) >> 1] = dw;
-          }
+      for (int e = 0; e < EPO; ++e) {
+        const int r = op * EPO + e;
+        if (r < 16) {
+          pe[r] = fast_exp2(SC[r]);
+          asm volatile("" : "+v"(pe[r]));
+        }
+        if (r >= 1 && r <= 16) {
+          de[r - 1] = pe[r - 1] * PC[r - 1];
+          asm volatile("" : "+v"(de[r - 1]));
+        }
+        if (r >= 2 && r <= 16 && !(r & 1)) {
+          unsigned pw = pack2(pe[r - 2], pe[r - 1]), dw = pack2(de[r - 2], de[r - 1]);
+          asm volatile("" : "+v"(pw), "+v"(dw));
+          pfw[(r - 2) >> 3][((r - 2) & 7) >> 1] = pw;
+          dsw[(r - 2) >> 3][((r - 2) & 7) >> 1] = dw;
         }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (!(RA_ABLATE_B & 8)) {
-      de[15] = pe[15] * PC[15];
-      pfw[1][3] = pack2(pe[14], pe[15]);
-      dsw[1][3] = pack2(de[14], de[15]);
-    }
-    RA_PROF_MARK(i, 4);
+    de[15] = pe[15] * PC[15];
+    pfw[1][3] = pack2(pe[14], pe[15]);
+    dsw[1][3] = pack2(de[14], de[15]);
   };
 
   // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
@@ -751,7 +720,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  RA_STAMP(5);
   if (pend_valid) {  // products of the last tile
     bf16x8 pf[2], dsf[2];
 #pragma unroll
@@ -763,9 +731,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     compute_dkdv(pf, dsf, s_q[0] + last * TILE_BYTES, s_do[0] + last * TILE_BYTES);
   }
   }  // query shards
-
-  RA_PROF_DUMP;
-  RA_STAMP(6);
   // ---- accumulate into the fp32 gradients owned by this key slab ------------------------------
   // All loads of an array are issued before the first value is needed: a load - add - store chain
   // per element would cost one memory round trip each, a hundred in a row with nothing to hide them.
@@ -799,7 +764,6 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     add_to(dkp, dk, a.sm_scale);
     add_to(dvp, dv, 1.0f);
   }
-  RA_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -829,8 +793,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   constexpr int ROWB = D * 2;
   constexpr int TILE_BYTES = kDqKeyTile * ROWB;
   constexpr int NBUF = 6;
-
-  RA_STAMP(0);
   __shared__ __attribute__((aligned(16))) char s_k[NBUF][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char s_v[NBUF][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) int s_seg[NBUF][kDqKeyTile];
@@ -905,7 +867,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     if (flags & RA_BIAS_PREFIX) q_pre = bs.q_pre[b * bs.q_pre_sb + qi_c];
     if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e;
   }
-  RA_PROFQ_DECL
   // ---- one pass of everything below per key/value shard ------------------------------------
   int kv_off = bs.kv_off;
   const bf16_t* k_ptr = a.k.ptr;
@@ -1154,10 +1115,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     }
     if (n > 2) issue_tile(tile_at(2, sbu), 2);  // its ids are stored at the top of iteration 0
   }
-  RA_STAMP(2);
   __builtin_amdgcn_s_waitcnt(0);
   __syncthreads();
-  RA_STAMP(3);
 
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
@@ -1191,7 +1150,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       if (needs_bias(kt0, segbit, cls)) prepare(s_a, kt0, segbit, cls, 0);
     }
   }
-  RA_STAMP(4);
   // dS^T(i-1), packed in pairs, waiting for its dQ^T product
   u32x4 dsw[2];
 #pragma unroll
@@ -1282,7 +1240,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     const char* kn = s_k[PH1];
     const char* vn = s_v[PH1];
     // operands of the dQ^T product come from tile i-1, visible since two barriers ago
-    RA_PROFQ_MARK(i, 1);
     bf16x8 frb[2 * DB];
 #pragma unroll
     for (int op = 0; op < PF; ++op) frb[op] = tr_frag(kp, op / DB, op % DB);
@@ -1291,7 +1248,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       __builtin_amdgcn_s_waitcnt(0x0f72);
       __syncthreads();
     }
-    RA_PROFQ_MARK(i, 2);
     bf16x8 dsf[2];
     dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
     dsf[1] = __builtin_bit_cast(bf16x8, dsw[1]);
@@ -1319,7 +1275,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 #pragma unroll
       for (int op = 0; op < PF; ++op) fra[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
     }
-    RA_PROFQ_MARK(i, 3);
     bf16x8 q0 = qf[0], do0 = dof[0];
     if (TIGHT) {
       q0 = s_q0[tid];
@@ -1376,7 +1331,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     }
     chain_links(2 * KS);      // the links that the last slots left over
     chain_links(2 * KS + 1);
-    RA_PROFQ_MARK(i, 4);
   };
 
   // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
@@ -1451,7 +1405,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  RA_STAMP(5);
   if (pend_valid) {  // product of the last tile
     bf16x8 dsf[2];
     dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
@@ -1459,9 +1412,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     compute_dq(dsf, s_k[0] + ((n - 1) % NBUF) * TILE_BYTES);
   }
   }  // key/value shards
-
-  RA_PROFQ_DUMP;
-  RA_STAMP(6);
   if (q_valid) {
     float* dq = a.dq + row * D + 4 * g;
 #pragma unroll
@@ -1474,7 +1424,6 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         *(f32x4*)(dq + 32 * db + 8 * bb) = t;
       }
   }
-  RA_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------

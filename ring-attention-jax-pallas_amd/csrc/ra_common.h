@@ -20,41 +20,6 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 #define RA_DEV __device__ __forceinline__
 
-// Optional in-kernel phase timing (build with -DRA_PROFILE): every wave accumulates, in scalar
-// registers, the cycles spent between consecutive marks; waves 0 and 4 of workgroup 0 write
-// the sums to g_prof[wave/4][segment] when the kernel ends.  Compiles to nothing otherwise.
-#ifdef RA_PROFILE
-__device__ unsigned int g_prof[2][16];
-#define RA_PROF_DECL unsigned int prof_seg[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long prof_t = __builtin_readcyclecounter();
-#define RA_PROF_MARK(iter, id)                                         \
-  do {                                                                 \
-    unsigned long long t_ = __builtin_readcyclecounter();              \
-    prof_seg[id] += (unsigned int)(t_ - prof_t);                       \
-    prof_t = t_;                                                       \
-  } while (0)
-#define RA_PROF_DUMP                                                   \
-  do {                                                                 \
-    if (blockIdx.x == 0 && (threadIdx.x & 255) == 0)                   \
-      for (int i_ = 0; i_ < 8; ++i_) g_prof[threadIdx.x >> 8][i_] = prof_seg[i_]; \
-  } while (0)
-#else
-#define RA_PROF_DECL
-#define RA_PROF_MARK(iter, id) do { } while (0)
-#define RA_PROF_DUMP do { } while (0)
-#endif
-
-// Optional wall-clock stamps of one workgroup in the middle of the grid (build with -DRA_STAMPS):
-// g_stamp[k] receives the 100 MHz counter when thread 0 of that workgroup passes RA_STAMP(k).
-#ifdef RA_STAMPS
-__device__ unsigned long long g_stamp[16];
-#define RA_STAMP(k)                                                                           \
-  do {                                                                                        \
-    if (threadIdx.x == 0 && blockIdx.x == gridDim.x / 2) g_stamp[k] = wall_clock64();         \
-  } while (0)
-#else
-#define RA_STAMP(k) do { } while (0)
-#endif
-
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 #define RA_NEG_INF (-__builtin_inff())
@@ -261,7 +226,7 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
         if (!(tb.flags & RA_BIAS_CAUSAL)) msk |= -rel >= tb.window;
       }
       if (tb.flags & RA_BIAS_SEGMENT) msk |= vs[c] != fixed_seg;
-      if (tb.flags & RA_BIAS_PREFIX) msk |= !(((vp[c] & fixed_pre) != 0) | (rel >= 0));
+      if (tb.flags & RA_BIAS_PREFIX) msk |= !(((vp[c] != 0) & (fixed_pre != 0)) | (rel >= 0));
       t[r] = msk ? RA_NEG_INF : x;
     }
   }

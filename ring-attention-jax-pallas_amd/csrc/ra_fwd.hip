@@ -11,15 +11,7 @@
 
 #include "ra_launch.h"
 
-#ifndef RA_ABLATE
-#define RA_ABLATE 0  // timing experiments only: bit mask of loop parts to leave out
-#endif
-
 namespace ra {
-
-#ifdef RA_CLOCK
-__device__ unsigned long long g_clock[2];  // timing experiments only: core cycles and 100 MHz ticks of workgroup 0
-#endif
 
 constexpr int kFwdThreads = 512;
 constexpr int kFwdRows = 256;   // query rows per workgroup
@@ -56,15 +48,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   const int wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);  // same value in a scalar register
   const int l32 = lane & 31, g = lane >> 5;
-#ifdef RA_CLOCK
-  // kept in LDS, the kernel has no scalar register to spare
-  __shared__ unsigned long long s_clock[2];
-  if (tid == 0) {
-    s_clock[0] = __builtin_readcyclecounter();
-    s_clock[1] = wall_clock64();
-  }
-#endif
-  RA_STAMP(0);
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   int hh, qt;
   decode_block(blockIdx.x, a.B * a.H, nqt, hh, qt);
@@ -117,7 +100,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e;
   }
   float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
-  RA_PROF_DECL
 
   // ---- one pass of everything below per key/value shard ------------------------------------
   int kv_off = bs.kv_off;
@@ -150,8 +132,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   const bool q_valid = qi < a.Lq;
   const int* kv_seg = (GENERAL && (flags & RA_BIAS_SEGMENT)) ? kv_seg_ptr + b * bs.kv_seg_sb : nullptr;
   const int* kv_pre = (GENERAL && (flags & RA_BIAS_PREFIX)) ? kv_pre_ptr + b * bs.kv_pre_sb : nullptr;
-
-  RA_STAMP(1);
   // ---- which key tiles does this workgroup visit ------------------------------------------
   const int ntiles = (a.Lk + kKeyTile - 1) / kKeyTile;
   const int q_rows_hi = min(q0 + kFwdRows, a.Lq) - 1;
@@ -294,7 +274,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   int sb_unused;
   // part t of the request for K tile ordinal j / V tile ordinal j (nothing if the tile does not exist)
   auto request_k = [&](int j, int t) {
-    if (j < n && t < NLD && !(RA_ABLATE & 1)) {
+    if (j < n && t < NLD) {
       const int k0 = tile_at(j, sb_unused) * kKeyTile;
       issue_part(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + (j & 3) * TILE_BYTES + wave_u * 8 * (D * 2), t);
       if (GENERAL && t == 0 && tid < kKeyTile) {
@@ -305,7 +285,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
   };
   auto request_v = [&](int j, int t) {
-    if (j < n && t < NLD && !(RA_ABLATE & 1)) {
+    if (j < n && t < NLD) {
       const int k0 = tile_at(j, sb_unused) * kKeyTile;
       issue_part(vbase, v_voff, a.v.sl, k0, RA_LDS_ADDR(&s_v[0][0]) + (j & 3) * TILE_BYTES + wave_u * 8 * (D * 2), t);
     }
@@ -336,7 +316,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // barrier k the tiles K_{k+1}, V_{k-1} (late waves) and V_k are read while K_{k+2}, K_{k+3},
   // V_{k+1}, V_{k+2} land: three K and four V tiles are live.
   const bool wave_on = qw < a.Lq;
-  RA_STAMP(2);
   // what barriers -3, -2, -1 would have requested
   if (n > 0) {
     issue_k(tile_at(0, sb_unused), 0);
@@ -352,10 +331,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     issue_k(tile_at(2, sb_unused), 2);
     store_ids(2);
   }
-  RA_STAMP(3);
   __builtin_amdgcn_s_waitcnt(0);  // tiles, carry and Q operands have landed
   __syncthreads();
-  RA_STAMP(4);
 
   constexpr int PF = 3;  // LDS operand fetches kept in flight ahead of the MFMA that uses them
 
@@ -389,11 +366,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
   constexpr int ROWB = D * 2;
   auto s_op_frag = [&](const char* kt, int op) {
-    if (RA_ABLATE & 32) return qf[op >> 1];
     return *(const bf16x8*)(kt + (32 * (op & 1)) * ROWB + koff[op >> 1]);
   };
   auto pv_op_frag = [&](unsigned vt, int op) {  // vt: byte offset of the tile buffer inside s_v
-    if (RA_ABLATE & 64) return qf[op % KS];
     const unsigned cofs = (32 * (op / (2 * DB)) + 16 * ((op / DB) & 1)) * ROWB;
     const lds_char* p0 = (const lds_char*)(uintptr_t)((unsigned)voff[op % DB][0] + (vt + cofs));
     const lds_char* p1 = (const lds_char*)(uintptr_t)((unsigned)voff[op % DB][1] + (vt + cofs));
@@ -518,7 +493,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (GENERAL || k == 0 || pending == 0) __builtin_amdgcn_s_waitcnt(0x0f70);
     else if (pending == NLD) __builtin_amdgcn_s_waitcnt(0x0f70 | NLD);
     else __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));
-    if (!(RA_ABLATE & 8)) __syncthreads();
+    __syncthreads();
   };
 
   // per-tile state handed from one iteration to the next
@@ -539,9 +514,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // one iteration; SC holds S(i) on entry, SN receives S(i+1)
   auto iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
     constexpr int PAR = decltype(parity)::value;  // i & 3, known at compile time
-    RA_PROF_MARK(i, 1);
     if (!late_half) sync(i);
-    RA_PROF_MARK(i, 2);
     const char* kt = s_k[(PAR + 1) & 3];
     const unsigned vt = PAR * TILE_BYTES;
     int nkt0 = 0, nsegbit = 0, ncls = 1;
@@ -558,8 +531,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const bool fused = cur_valid && nxt_valid && !cur_scaled;
     if (cur_valid) update_reference(cur_mx);
     const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
-
-    RA_PROF_MARK(i, 3);
     if (fused) {
       // ---- fused path: S(i+1) MFMAs with the exp2 / sum / pack of tile i in their shadow -------
       float rs0 = 0.f, rs1 = 0.f;
@@ -577,12 +548,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 #pragma unroll
         for (int op = 0; op < 2 * KS; ++op) {
           if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
-          if (!(RA_ABLATE & 16)) SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
-          else SN[op & 1][op >> 1] += (float)fr[op][0];
+          SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
           if (op == (2 * KS) / 4) request_k(i + 3, 0);
           if (op == (2 * KS) * 3 / 4) request_k(i + 3, 1);
 #pragma unroll
-          for (int e = 0; e < ((RA_ABLATE & 2) ? 0 : EPO); e += 2) {
+          for (int e = 0; e < EPO; e += 2) {
             const int el = op * EPO + e;  // 0..31 over (kb, r)
             const int kb = el >> 4, r = el & 15;
             const float p0 = fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
@@ -606,7 +576,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         }
       }
       l_run += rs0 + rs1;
-      RA_PROF_MARK(i, 4);
       if (late_half) sync(i + 1);
       // ---- O += P(i) V_i with the row maximum of S(i+1) in the shadow ---------------------------
       {
@@ -619,8 +588,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 #pragma unroll
         for (int op = 0; op < 4 * DB; ++op) {
           if (op + PF < 4 * DB) fr[op + PF] = pv_op_frag(vt, op + PF);
-          if (!(RA_ABLATE & 4)) oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
-          else oacc[op % DB][op / DB] += (float)fr[op][0] * (float)pfrag[op / DB][0];
+          oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
           if (op == (4 * DB) / 4) request_v(i + v_ahead, 0);
           if (op == (4 * DB) * 3 / 4) request_v(i + v_ahead, 1);
 #pragma unroll
@@ -633,7 +601,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         }
         nxt_mx = half_max(fmaxf(mx0, mx1)) * a.scale2;
       }
-      RA_PROF_MARK(i, 5);
     } else {
       // ---- generic path (first / last / masked / biased tiles): same work, not interleaved -----
       request_k(i + 3, 0);
@@ -670,7 +637,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       if (cur_valid) compute_pv(pfrag, vt);
       if (nxt_valid && !nxt_scaled) nxt_mx = raw_rowmax(SN);
     }
-    RA_PROF_MARK(i, 6);
     if (nxt_scaled) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, (i + 1) & 3);
     if (i + 3 < n) store_ids((i + 3) & 3);
     cur_valid = nxt_valid;
@@ -698,15 +664,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   auto plain_iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
     constexpr int PAR = decltype(parity)::value;
     constexpr int PF = TIGHT ? 2 : 3;  // these variants have four registers less to spare
-    RA_PROF_MARK(i, 1);
     if (!late_half) sync_plain();
-    RA_PROF_MARK(i, 2);
     const char* kt = s_k[(PAR + 1) & 3];
     const unsigned vt = PAR * TILE_BYTES;
     update_reference(cur_mx);
     const float neg_m = -m_run;  // finite: the current tile has unmasked scores
     const unsigned v_dst = v_dst0 + (late_half ? ((PAR + 3) & 3) : ((PAR + 2) & 3)) * TILE_BYTES;
-    RA_PROF_MARK(i, 3);
     // ---- S(i+1) MFMAs, then O += P(i) V_i, with the softmax arithmetic of tile i and the row
     // maximum of S(i+1) in their shadow.  The chain of a pair of scores (scale and shift, exp2,
     // pack, row sum) is spread over four consecutive MFMA slots, one link per slot, so that no
@@ -783,7 +746,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       }
     }
     k_run += (long long)kKeyTile * a.k.sl;
-    RA_PROF_MARK(i, 4);
     if (late_half) sync_plain();
     {
       bf16x8 fr[NOPB];
@@ -812,7 +774,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       cur_mx = half_max(fmaxf(mx0, mx1)) * a.scale2;
     }
     v_run += (long long)kKeyTile * a.v.sl;
-    RA_PROF_MARK(i, 5);
   };
 
   if (late_half) {
@@ -879,18 +840,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
     if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
   }
-  RA_STAMP(5);
   if (!late_half) sync(n);  // both halves pass the same number of barriers
-  RA_STAMP(6);
   }  // key/value shards
-
-  RA_PROF_DUMP;
-#ifdef RA_CLOCK
-  if (blockIdx.x == 0 && tid == 0) {
-    g_clock[0] = __builtin_readcyclecounter() - s_clock[0];
-    g_clock[1] = wall_clock64() - s_clock[1];
-  }
-#endif
   // ---- merge this step into the carry ---------------------------------------------------------
   // o = o_in 2^(m_in - m_out) + o_step 2^(m_run - m_out) l_step / lr_step,  l likewise with the
   // exact sum, m_out = exact maximum over carry and step.
@@ -924,7 +875,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       }
     }
   }
-  RA_STAMP(7);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -955,9 +905,11 @@ __global__ void fwd_finalize_kernel(const float* o, const float* m, const float*
   const int b = (int)(row / ((long long)Lq * H));
   const float lv = l[row];
   f32x4 x = *(const f32x4*)(o + row * D + 4 * c);
-  OutT* dst = out + b * sb + h * sh + (long long)li * sl + 4 * c;
+  typedef __attribute__((ext_vector_type(4))) OutT out4;
+  out4 y;
 #pragma unroll
-  for (int e = 0; e < 4; ++e) dst[e] = (OutT)(x[e] / lv);
+  for (int e = 0; e < 4; ++e) y[e] = (OutT)(x[e] / lv);
+  *(out4*)(out + b * sb + h * sh + (long long)li * sl + 4 * c) = y;
   if (c == 0) lse[row] = m[row] + logf(lv);
 }
 

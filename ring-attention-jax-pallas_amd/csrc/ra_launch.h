@@ -66,7 +66,6 @@ hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long lon
 hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStream_t stream);
 hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream);
 hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QShardList& shards, int D, int mode, hipStream_t stream);
-hipError_t launch_mfma_rate(float* sink, int blocks, int iters, int random, hipStream_t stream);
 hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl,
                                int B, int H, int L, int D, hipStream_t stream);
 

@@ -1,8 +1,9 @@
+// Benchmark-only library (libringattn_probe.so), not part of the block-step ABI.
 // Diagnostic: the bf16 MFMA rate this GPU sustains with nothing but matrix instructions in flight.
 // The published dense peak assumes the maximum clock; under a full matrix load with operands
 // that toggle like real data the clock settles lower, so the rate measured here is the ceiling
 // any kernel made of v_mfma_f32_32x32x16_bf16 can approach on this board.
-#include "ra_launch.h"
+#include "ra_common.h"
 
 namespace ra {
 
@@ -48,10 +49,16 @@ __global__ __launch_bounds__(256) void mfma_rate_kernel(float* sink, int iters) 
   sink[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
-hipError_t launch_mfma_rate(float* sink, int blocks, int iters, int random, hipStream_t stream) {
-  if (random) hipLaunchKernelGGL((mfma_rate_kernel<1>), dim3(blocks), dim3(256), 0, stream, sink, iters);
-  else hipLaunchKernelGGL((mfma_rate_kernel<0>), dim3(blocks), dim3(256), 0, stream, sink, iters);
-  return hipGetLastError();
-}
-
 }  // namespace ra
+
+// Launches `blocks` workgroups of four waves (one per SIMD) that each issue iters x 8 independent
+// v_mfma_f32_32x32x16_bf16 and nothing else; the caller times the launch and divides
+// blocks * 4 * iters * 8 * 32768 FLOP by it.  `sink` receives blocks * 256 floats.  Returns 0, -1
+// for bad arguments or the HIP error code of the launch.
+extern "C" int ra_probe_mfma_rate(float* sink, int blocks, int iters, int random_operands, void* stream) {
+  if (!sink || blocks <= 0 || blocks > 65536 || iters <= 0 || (iters % 4)) return -1;
+  hipStream_t st = (hipStream_t)stream;
+  if (random_operands) hipLaunchKernelGGL((ra::mfma_rate_kernel<1>), dim3(blocks), dim3(256), 0, st, sink, iters);
+  else hipLaunchKernelGGL((ra::mfma_rate_kernel<0>), dim3(blocks), dim3(256), 0, st, sink, iters);
+  return (int)hipGetLastError();
+}

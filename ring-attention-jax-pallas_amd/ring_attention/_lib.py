@@ -79,7 +79,6 @@ EXPORTS = {
     "ra_step_is_skippable": (C.c_int, [C.POINTER(RaBias), C.c_int32, C.c_int32]),
     "ra_fwd_step_check": (C.c_int, [C.POINTER(RaFwdStepParams)]),
     "ra_bwd_step_check": (C.c_int, [C.POINTER(RaBwdStepParams)]),
-    "ra_probe_mfma_rate": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
 }
 
 _lib = None

@@ -15,8 +15,10 @@ The per-token arrays keep the reference's kwarg names (ring.py:411-420):
 ``q_segment_ids`` / ``kv_segment_ids``, ``q_positions`` / ``kv_positions``,
 ``q_prefix_mask`` / ``kv_prefix_mask``; the q-side ones go into ``bias_q_kwargs`` and the
 kv-side ones into ``bias_kv_kwargs``.  Positions are optional: when absent a token's
-position is its index in the global sequence; when given they must be consecutive inside
-every shard (the kernels take one offset per shard).
+position is its index in the global sequence.  Positions that are consecutive inside every
+shard and equal across the batch cost nothing (the kernels take one offset per shard); any other
+positions are honoured by materialising the terms per ring step as a dense block, the slow path
+of a callable ``bias_fn``.
 """
 from __future__ import annotations
 

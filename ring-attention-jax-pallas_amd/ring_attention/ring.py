@@ -315,29 +315,47 @@ class _RingPlan:
                 self.kv_pre = ids(kv_kwargs.get("kv_prefix_mask"), Sk, "kv_prefix_mask")
                 if self.q_pre is None or self.kv_pre is None:
                     raise ValueError("prefix bias needs q_prefix_mask and kv_prefix_mask")
-            if fn.needs_positions:
-                qp, kp = q_kwargs.get("q_positions"), kv_kwargs.get("kv_positions")
-                if qp is not None:
-                    self.q_off = self._offsets(qp, Sq, self.Lq, "q_positions")
-                if kp is not None:
-                    self.kv_off = self._offsets(kp, Sk, self.Lk, "kv_positions")
             if fn.alibi_slopes is not None:
                 if fn.alibi_slopes.numel() != self.H:
                     raise ValueError("alibi slopes must have one entry per head")
-                self.fn = BiasFn(fn.causal, fn.window, fn.segments, fn.prefix,
-                                 fn.alibi_slopes.to(device=dev, dtype=torch.float32).contiguous())
+                self.fn = fn = BiasFn(fn.causal, fn.window, fn.segments, fn.prefix,
+                                      fn.alibi_slopes.to(device=dev, dtype=torch.float32).contiguous())
+            if fn.needs_positions:
+                qp, kp = q_kwargs.get("q_positions"), kv_kwargs.get("kv_positions")
+                q_off = self.q_off if qp is None else self._offsets(qp, Sq, self.Lq, "q_positions")
+                kv_off = self.kv_off if kp is None else self._offsets(kp, Sk, self.Lk, "kv_positions")
+                if q_off is None or kv_off is None:
+                    # Arbitrary positions (the reference compares kv_positions <= q_positions element
+                    # by element, ring.py:396): the kernels take one offset per shard, so the terms
+                    # are materialised per ring step from the position arrays and streamed as a
+                    # dense block, like a callable bias_fn.
+                    def full(t, S):
+                        if t is None:
+                            t = torch.arange(S, device=dev)[None].expand(self.B, S)
+                        return t.to(device=dev, dtype=torch.int64)
+                    self.callable = _positional_bias_callable(fn)
+                    self.fn = None
+                    self.q_kw = {"q_positions": full(qp, Sq)}
+                    self.kv_kw = {"kv_positions": full(kp, Sk)}
+                    for kw, name, t in ((self.q_kw, "q_segment_ids", self.q_seg), (self.kv_kw, "kv_segment_ids", self.kv_seg),
+                                        (self.q_kw, "q_prefix_mask", self.q_pre), (self.kv_kw, "kv_prefix_mask", self.kv_pre)):
+                        if t is not None:
+                            kw[name] = t
+                    return
+                self.q_off, self.kv_off = q_off, kv_off
 
     def _offsets(self, pos, S, L, name):
-        """Positions must be consecutive inside each shard and equal across the batch."""
+        """One position offset per shard if the positions are consecutive inside every shard and
+        equal across the batch (what the in-kernel terms take); None otherwise."""
         if tuple(pos.shape) != (self.B, S):
             raise ValueError(f"{name} must have shape {(self.B, S)}, got {tuple(pos.shape)}")
         pos = pos.to(torch.int64)
         starts = pos[:, ::L]
         expect = (starts[:, :, None] + torch.arange(L, device=pos.device)[None, None, :]).reshape(self.B, S)
         if not torch.equal(expect, pos) or not bool((starts == starts[:1]).all()):
-            raise NotImplementedError(
-                f"{name}: the kernels take one position offset per shard, so positions must be "
-                "consecutive inside every shard and identical across the batch")
+            return None
+        if int(starts.min()) < 0 or int(starts.max()) + L > (1 << 30):
+            return None  # outside the offset range of the C ABI
         return [int(x) for x in starts[0].tolist()]
 
     def live_steps(self, qs: Optional[int], ks: Optional[int]) -> int:
@@ -375,6 +393,32 @@ class _RingPlan:
             None if self.kv_seg is None else self.kv_seg[:, sl_k],
             None if self.q_pre is None else self.q_pre[:, sl_q],
             None if self.kv_pre is None else self.kv_pre[:, sl_k])
+
+
+def _positional_bias_callable(fn: BiasFn):
+    """The terms of ``fn`` as a dense-bias callable of explicit per-token positions: the mask
+    builder of the reference (ring.py:376-409: segments ``:388-391``, causal ``kv_pos <= q_pos``
+    ``:393-397``, prefix-LM ``:399-406``, ``where(mask, 0, -inf)[:, None]`` ``:408-409``) plus the
+    window and ALiBi terms, for positions that one offset per shard cannot express."""
+    def bias_fn(q_positions, kv_positions, q_segment_ids=None, kv_segment_ids=None, q_prefix_mask=None,
+                kv_prefix_mask=None):
+        rel = q_positions[:, :, None] - kv_positions[:, None, :]  # [b, lq, lk]
+        mask = torch.ones_like(rel, dtype=torch.bool)
+        if fn.segments:
+            mask &= q_segment_ids[:, :, None] == kv_segment_ids[:, None, :]
+        if fn.causal:
+            mask &= rel >= 0
+        if fn.window is not None:
+            mask &= (rel < fn.window) if fn.causal else (rel.abs() < fn.window)
+        if fn.prefix:
+            mask &= ((q_prefix_mask[:, :, None] != 0) & (kv_prefix_mask[:, None, :] != 0)) | (rel >= 0)
+        bias = torch.zeros(mask.shape, dtype=torch.float32, device=mask.device)
+        bias.masked_fill_(~mask, float("-inf"))
+        bias = bias[:, None]
+        if fn.alibi_slopes is not None:
+            bias = bias - fn.alibi_slopes.to(bias.device)[None, :, None, None] * rel.abs()[:, None].to(torch.float32)
+        return bias
+    return bias_fn
 
 
 def _shard_bhld(x, s, L):

@@ -107,6 +107,37 @@ def test_bwd_step_rejects_bad_params_without_a_gpu(lib):
     assert lib.ra_fwd_finalize(0x10, 0x10, 0x10, 0x10, 5, 8, 8, 8, 0x10, 1, 1, 1, 64, None) == -7
 
 
+def test_finalize_entry_points_check_alignment_without_a_gpu(lib):
+    # ra_fwd_finalize stores four elements at a time: out must be aligned to 8 (bf16) / 16 (fp32) bytes
+    ok = (0x1000, 0x1000, 0x1000)
+    assert lib.ra_fwd_finalize(*ok, 0x2004, _lib.RA_DTYPE_BF16, 128, 128, 128, 0x3000, 1, 1, 4, 64, None) == -4
+    assert b"aligned" in lib.ra_last_error()
+    assert lib.ra_fwd_finalize(*ok, 0x2008, _lib.RA_DTYPE_F32, 128, 128, 128, 0x3000, 1, 1, 4, 64, None) == -4
+    assert lib.ra_fwd_finalize(0x1004, 0x1000, 0x1000, 0x2000, _lib.RA_DTYPE_F32, 128, 128, 128, 0x3000,
+                               1, 1, 4, 64, None) == -4
+    assert lib.ra_fwd_finalize(*ok, 0x2000, _lib.RA_DTYPE_F32, 130, 128, 128, 0x3000, 1, 1, 4, 64, None) == -4
+    # ra_bwd_finalize loads 16 bytes of fp32 and stores 8 bytes of bf16 at a time
+    assert lib.ra_bwd_finalize(0x1000, 0x2004, 128, 128, 128, 1, 1, 4, 64, None) == -4
+    assert b"8-byte" in lib.ra_last_error()
+    assert lib.ra_bwd_finalize(0x1008, 0x2000, 128, 128, 128, 1, 1, 4, 64, None) == -4
+    assert lib.ra_bwd_finalize(0x1000, 0x2000, 128, 126, 128, 1, 1, 4, 64, None) == -4
+
+
+def test_grids_beyond_the_launch_limit_are_rejected(lib):
+    # B*H*ceil(L/128) workgroups must fit a 31-bit grid dimension: a larger launch would be cut short
+    p = _good_fwd()
+    p.B, p.H, p.Lq = 1 << 10, 1 << 10, 1 << 22      # 2^20 heads x 2^15 tiles = 2^35 workgroups
+    assert lib.ra_fwd_step_check(C.byref(p)) == -2 and b"grid" in lib.ra_last_error()
+    p.Lq, p.Lk = 64, 1 << 22                          # the key side counts as well (dK/dV grid)
+    assert lib.ra_fwd_step_check(C.byref(p)) == -2
+    b = _good_bwd()
+    b.B, b.H, b.Lk = 1 << 10, 1 << 10, 1 << 22
+    assert lib.ra_bwd_step_check(C.byref(b)) == -2
+    p = _good_fwd()
+    p.B, p.H, p.Lq = 1 << 10, 1 << 10, 1 << 17      # 2^30 workgroups: still fine
+    assert lib.ra_fwd_step_check(C.byref(p)) == 0
+
+
 @pytest.mark.parametrize("flags,window", [(1, 0), (3, 7), (2, 7), (3, 64), (2, 1), (0, 0), (8, 0)])
 def test_step_is_skippable_matches_brute_force(lib, flags, window):
     Lq, Lk = 16, 24

@@ -1,7 +1,10 @@
 """GPU parity tests: the HIP kernels (through the C ABI) against the CPU oracle on the same
 seeded inputs.  Tolerances: forward output max-abs error <= 1e-2 and
 logsumexp <= 1e-3 for bf16 inputs against the fp64 oracle on the same bf16-rounded values,
-dq/dk/dv relative error <= 2e-2 (max|diff| / max|ref| and Frobenius)."""
+dq/dk/dv relative error <= 2e-2 (max|diff| / max|ref| and Frobenius).  Where outputs are small
+(long rows, N(0, 0.5^2) inputs) the absolute bound alone would let a large relative error
+through, so the output also has to stay within OUT_REL of the largest reference value of its
+(batch, head)."""
 import glob
 import math
 import os
@@ -17,6 +20,15 @@ from ring_attention import ring as rr
 pytestmark = pytest.mark.gpu
 
 OUT_TOL, LSE_TOL, GRAD_TOL = 1e-2, 1e-3, 2e-2
+OUT_REL = 1e-2  # max|out - ref| over a (batch, head) / max|ref| over the same (batch, head)
+
+
+def _out_rel(out, want):
+    """Largest max|diff| / max|ref| over the (batch, head) slices of [b, l, h, d] arrays (NaN rows
+    of the reference, fully masked queries, left out)."""
+    d = np.where(np.isnan(want), 0.0, np.abs(out - want))
+    ref = np.where(np.isnan(want), 0.0, np.abs(want))
+    return float((d.max(axis=(1, 3)) / np.maximum(ref.max(axis=(1, 3)), 1e-30)).max())
 
 
 def _dev(x, device, dtype=None):
@@ -61,14 +73,31 @@ def _check(device, name, B, Sq, Sk, H, D, n, fn=None, ofn=None, qkw=None, kvkw=N
     want, want_lse = R.mha_dense(q, k, v, bias)
     np.testing.assert_array_equal(np.isnan(out), np.isnan(want))
     ok = ~np.isnan(want)
-    assert np.abs(out - want)[ok].max() <= OUT_TOL
+    e_out, e_rel = np.abs(out - want)[ok].max(), _out_rel(out, want)
     okl = np.isfinite(want_lse)
     np.testing.assert_array_equal(np.isneginf(lse), np.isneginf(want_lse))
-    assert np.abs(lse[okl] - want_lse[okl]).max() <= LSE_TOL
-    if grads and ok.all():
+    e_lse = np.abs(lse[okl] - want_lse[okl]).max()
+    worst = {"out": e_out, "out_rel": e_rel, "lse": e_lse}
+    assert e_out <= OUT_TOL and e_rel <= OUT_REL and e_lse <= LSE_TOL, worst
+    if grads:
+        # Queries that see no key (NaN output, ring.py:134-135) must contribute nothing to dk / dv;
+        # the reference gradients are those of the attention over the live queries only (a dead
+        # row with a zero bias row and a zero dO row adds exactly nothing), and dq is compared on
+        # the live rows.
+        live = ok.all(axis=(2, 3))  # [b, lq]
+        if not live.all():
+            do = np.where(live[:, :, None, None], do, 0.0)
+            bias = np.where(live[:, None, :, None], bias, 0.0)
         for got, ref, nm in zip(g, R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
+            if nm == "dq":
+                got, ref = got[live], ref[live]
+            else:
+                assert np.isfinite(got).all(), nm
             mx, fro = _rel(got, ref)
+            worst[nm] = max(mx, fro)
             assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+    print("[parity]   worst: " + " ".join(f"{a} {b:.2e}" for a, b in worst.items()), flush=True)
+    return worst
 
 
 # ---- the reference's own test shapes (ring_test.py:48-53, :104-111), 8 shards, B=2 -------------
@@ -185,6 +214,48 @@ def test_prefix_lm(device):
     _check(device, "prefix+segments", 2, 512, 512, 2, 128, 4, ra.prefix_lm_bias() + ra.segment_bias(),
            R.make_bias_fn(use_prefix=True, use_segments=True),
            {"q_prefix_mask": pm, "q_segment_ids": seg}, {"kv_prefix_mask": pm, "kv_segment_ids": seg})
+
+
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_ring_self_attention_prefix_lm(device, impl):
+    """ring_self_attention(prefix_mask=..., positions=...) (ring.py:399-406): bidirectional inside
+    the prefix, causal after it, with document ids on top; forward and gradients."""
+    B, S, H, D, n = 2, 1024, 2, 128, 4
+    q, k, v, do = R.make_inputs(31, B, S, S, H, D)
+    pos = np.broadcast_to(np.arange(S), (B, S)).copy()
+    pm = (np.arange(S)[None, :] < np.array([[333], [700]])).astype(np.int32) * 7  # any non-zero value marks the prefix
+    seg = np.sort(np.random.default_rng(31).integers(0, 3, (B, S)), axis=1).astype(np.int32)
+    print(f"[parity] ring_self_attention prefix-LM impl={impl}", flush=True)
+    tq, tk, tv = (_dev(x, device, torch.bfloat16).requires_grad_(True) for x in (q, k, v))
+    out = ra.ring_self_attention(tq, tk, tv, ra.RingAxis("sp", n), None, segment_ids=_dev(seg, device),
+                                 positions=_dev(pos, device), prefix_mask=_dev(pm, device), block_impl=impl)
+    out.float().backward(_dev(do, device, torch.float32))
+    torch.cuda.synchronize()
+    bias = R.make_bias_fn(use_prefix=True, use_segments=True)(
+        q_segment_ids=seg, kv_segment_ids=seg, q_positions=pos, kv_positions=pos,
+        q_prefix_mask=(pm != 0).astype(np.int32), kv_prefix_mask=(pm != 0).astype(np.int32))
+    want, _ = R.mha_dense(q, k, v, bias)
+    # the public entry point returns bf16 for bf16 inputs: its rounding (2^-9 relative) comes on top
+    assert np.abs(out.detach().float().cpu().numpy() - want).max() <= OUT_TOL + 2.0 ** -9 * np.abs(want).max()
+    for t, ref, nm in zip((tq, tk, tv), R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
+        mx, fro = _rel(t.grad.float().cpu().numpy(), ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+
+
+def test_arbitrary_positions(device):
+    """Positions that no per-shard offset can express (strided, shuffled inside a shard, different
+    in every batch row) follow the reference's element-wise rule kv_positions <= q_positions
+    (ring.py:393-397) through the dense-block path."""
+    B, S, n = 2, 512, 4
+    rng = np.random.default_rng(17)
+    pos = np.stack([rng.permutation(S) * 3, np.arange(S)[::-1].copy()]).astype(np.int64)
+    seg = rng.integers(0, 2, (B, S)).astype(np.int32)
+    _check(device, "arbitrary-positions causal+segments", B, S, S, 2, 64, n, ra.causal_bias() + ra.segment_bias(),
+           R.make_bias_fn(causal=True, use_segments=True), {"q_positions": pos, "q_segment_ids": seg},
+           {"kv_positions": pos, "kv_segment_ids": seg})
+    sl = R.alibi_slopes(2)
+    _check(device, "arbitrary-positions window+alibi", B, S, S, 2, 128, n, ra.sliding_window_bias(200) + ra.alibi_bias(sl),
+           R.make_bias_fn(causal=True, window=200, alibi=sl), {"q_positions": pos}, {"kv_positions": pos})
 
 
 def test_shard_positions_with_offsets(device):
@@ -567,12 +638,11 @@ def test_ring_replays_from_a_captured_graph(device, impl):
             assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3])
-def test_random_configurations(device, seed):
-    """Seeded random shapes (ragged shard lengths, cross attention, padded head dims, ring sizes
-    1..8) and bias combinations, each through both launch schemes, against the dense oracle."""
+def _random_cases(seed, count):
+    """The seeded sweep generator: ragged shard lengths, cross attention, padded head dims, ring
+    sizes 1..8 and nine bias combinations."""
     rng = np.random.default_rng(seed)
-    for case in range(12):
+    for case in range(count):
         B, H = int(rng.integers(1, 3)), int(rng.choice([1, 2, 4]))
         D = int(rng.choice([64, 128, 32, 96]))
         n = int(rng.choice([1, 2, 3, 4, 8]))
@@ -608,9 +678,67 @@ def test_random_configurations(device, seed):
         }[kind]
         std = float(rng.choice([0.5, 1.0]))
         data_seed = int(rng.integers(1 << 30))
+        yield case, kind, dict(B=B, Sq=Sq, Sk=Sk, H=H, D=D, n=n, fn=fn, ofn=ofn, qkw=qkw, kvkw=kvkw, std=std,
+                               seed=data_seed)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_configurations(device, seed):
+    """Seeded random shapes and bias combinations, each through both launch schemes, against the
+    dense oracle."""
+    for case, kind, kw in _random_cases(seed, 12):
         for impl in ("hip", "hip_fused"):
-            _check(device, f"random {seed}.{case} {kind}", B, Sq, Sk, H, D, n, fn, ofn, qkw, kvkw, std=std,
-                   seed=data_seed, impl=impl)
+            _check(device, f"random {seed}.{case} {kind}", impl=impl, **kw)
+
+
+# The cases of the seed-0 sweep with shard lengths off the tile grid (300, 520, 100 queries;
+# 250, 400, 96 keys) that an earlier hand-run sweep reported above tolerance.  That run drew its
+# inputs from N(0, 2^2): scores with a standard deviation of 4 and outputs up to 8.5, where the
+# half-ulp of a bf16 probability (2^-9 relative) alone is worth 1e-2 on the output.  At the
+# amplitudes of the benchmark configurations (N(0, 1) and N(0, 0.5^2)) every one of them is
+# within tolerance; at N(0, 2^2) the output stays within 2.5e-3 of its largest value.
+_SEED0_RAGGED = (9, 20, 21, 32, 55, 58, 67)
+
+
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_seed0_ragged_sweep_cases(device, impl):
+    worst = {}
+    for case, kind, kw in _random_cases(0, max(_SEED0_RAGGED) + 1):
+        if case not in _SEED0_RAGGED:
+            continue
+        for std in (0.5, 1.0):
+            got = _check(device, f"seed-0 sweep case {case} {kind} std={std}", impl=impl, **{**kw, "std": std})
+            for a, b in got.items():
+                worst[a] = max(worst.get(a, 0.0), b)
+    print("[parity] seed-0 ragged cases, worst over all: " + " ".join(f"{a} {b:.2e}" for a, b in worst.items()),
+          flush=True)
+
+
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_seed0_ragged_sweep_cases_at_four_times_the_score_spread(device, impl):
+    """The same cases with N(0, 2^2) inputs (what the hand-run sweep used): outside the amplitude
+    the absolute tolerances are stated for, so the output is held to a relative bound, and the
+    logsumexp and the gradients to theirs."""
+    for case, kind, kw in _random_cases(0, max(_SEED0_RAGGED) + 1):
+        if case not in _SEED0_RAGGED:
+            continue
+        print(f"[parity] seed-0 sweep case {case} {kind} std=2.0 impl={impl}", flush=True)
+        q, k, v, do = R.make_inputs(kw["seed"], kw["B"], kw["Sq"], kw["Sk"], kw["H"], kw["D"], std=2.0)
+        out, lse, g = _run_hip(device, q, k, v, do, kw["n"], kw["fn"], kw["qkw"], kw["kvkw"], impl=impl)
+        oq, okv = dict(kw["qkw"]), dict(kw["kvkw"])
+        bias = None
+        if kw["ofn"] is not None:
+            oq.setdefault("q_positions", np.broadcast_to(np.arange(kw["Sq"]), (kw["B"], kw["Sq"])))
+            okv.setdefault("kv_positions", np.broadcast_to(np.arange(kw["Sk"]), (kw["B"], kw["Sk"])))
+            bias = kw["ofn"](**oq, **okv)
+        want, want_lse = R.mha_dense(q, k, v, bias)
+        assert not np.isnan(want).any()
+        rel = np.abs(out - want).max() / np.abs(want).max()
+        assert rel <= 2.5e-3, (case, rel)
+        assert np.abs(lse - want_lse).max() <= LSE_TOL
+        for got, ref, nm in zip(g, R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
+            mx, fro = _rel(got, ref)
+            assert mx <= 3e-2 and fro <= 3e-2, (case, nm, mx, fro)
 
 
 def test_delta_kernel(device):
@@ -656,14 +784,57 @@ def test_fp32_and_fp16_inputs_are_cast(device):
 
 
 # ---- benchmark configs at full size -------------------------------------------------------------------------
-def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, bias_col, qkw=None, kvkw=None,
-                   impl="hip"):
-    """Full-size run on the GPU; the oracle is evaluated densely (fp64) on sampled query rows
-    (out, lse, dq) and sampled key columns (dk, dv; these use the GPU's lse/out for the other
-    rows, which the row samples vouch for), plus two exact invariants of softmax attention."""
-    print(f"[parity] {name}: B={B} H={H} D={D} S={S} ring={n}", flush=True)
-    gen = torch.Generator(device=device); gen.manual_seed(0)
-    mk = lambda s: (torch.randn((B, S, H, D), generator=gen, device=device) * s).to(torch.bfloat16)
+def _dense_reference_on_device(Q, K, V, DO, scale, bias_rows, chunk=1024):
+    """The dense closed form softmax(Q K^T * scale + bias) V and its analytic gradients
+    (oracle mha_dense / mha_dense_grads, ring.py:142-155) for ONE (batch, head), evaluated in fp64
+    with torch matrix products on the device, a chunk of query rows at a time.  ``bias_rows(i0, i1)``
+    returns the additive bias rows [i1 - i0, Sk] (fp64, -inf masks).  Independent of the HIP
+    kernels: nothing of their output enters.  Returns out, lse, dq, dk, dv."""
+    Sq, Sk = Q.shape[0], K.shape[0]
+    out, lse = torch.empty_like(Q), torch.empty(Sq, dtype=torch.float64, device=Q.device)
+    dq, dk, dv = torch.empty_like(Q), torch.zeros_like(K), torch.zeros_like(V)
+    for i0 in range(0, Sq, chunk):
+        i1 = min(i0 + chunk, Sq)
+        s = (Q[i0:i1] @ K.T) * scale + bias_rows(i0, i1)
+        m = s.max(dim=1, keepdim=True).values
+        p = torch.exp(s - m)
+        l = p.sum(dim=1, keepdim=True)
+        p /= l
+        lse[i0:i1] = (m + torch.log(l))[:, 0]
+        o = p @ V
+        out[i0:i1] = o
+        g = DO[i0:i1]
+        dv += p.T @ g
+        dp = g @ V.T
+        ds = p * (dp - (o * g).sum(dim=1, keepdim=True)) * scale
+        dq[i0:i1] = ds @ K
+        dk += ds.T @ Q[i0:i1]
+    return out, lse, dq, dk, dv
+
+
+def _full_size_check(device, name, B, H, D, S, n, fn, std, bias_rows_t, bias_row_np, qkw=None, kvkw=None,
+                     impl="hip", heads=None, n_rows=256):
+    """One benchmark configuration at full size through the HIP path, inputs as bench.py makes them
+    (the oracle's make_inputs stream, seed 0).  Checked, for every batch and the chosen heads:
+      * EVERY row of out, lse, dq, dk, dv against the dense fp64 closed form evaluated on the
+        device by torch (which never sees a kernel output);
+      * that torch evaluation itself against the numpy oracle formulas on n_rows sampled query
+        rows per head - row 0, every shard boundary -1 / +0 / +1, the last row, random rows -
+        which ties the full-size reference to the oracle;
+      * two invariants of softmax attention on all heads, with relative slack only."""
+    print(f"[parity] {name}: B={B} H={H} D={D} S={S} ring={n} impl={impl}", flush=True)
+    rng = np.random.default_rng(0)
+
+    def mk(sd):
+        t = torch.empty(B * S * H * D, device=device, dtype=torch.bfloat16)
+        piece = 1 << 26
+        for a0 in range(0, t.numel(), piece):
+            x = rng.standard_normal(min(piece, t.numel() - a0), dtype=np.float32)
+            if sd != 1.0:
+                x *= np.float32(sd)
+            t[a0:a0 + x.size] = torch.from_numpy(x).to(device).to(torch.bfloat16)
+        return t.view(B, S, H, D)
+
     q, k, v, do = mk(std), mk(std), mk(std), mk(1.0)
     q.requires_grad_(True); k.requires_grad_(True); v.requires_grad_(True)
     out, lse = ra.ring_attention_with_lse(q, k, v, n, bias_fn=fn, bias_q_kwargs=qkw, bias_kv_kwargs=kvkw,
@@ -672,76 +843,84 @@ def _sampled_check(device, name, B, H, D, S, n, fn, std, rows, cols, bias_row, b
     torch.cuda.synchronize()
     scale = 1 / math.sqrt(D)
     # invariants (exact in real arithmetic whenever every query sees at least one key):
-    #   sum_j dv_j = sum_i do_i          (rows of P sum to one)
-    #   <q, dq> = <k, dk>                (both equal sum_ij ds_ij s_ij / scale ... per head)
-    dv_sum = v.grad.float().sum(dim=1); do_sum = do.float().sum(dim=1)
-    assert (dv_sum - do_sum).abs().max().item() <= 2e-2 * do_sum.abs().max().item() + 0.5
-    qdq = (q.detach().float() * q.grad.float()).sum(dim=(1, 3)); kdk = (k.detach().float() * k.grad.float()).sum(dim=(1, 3))
-    assert (qdq - kdk).abs().max().item() <= 2e-2 * qdq.abs().max().item() + 1.0
-    b = 0
-    heads = sorted({0, H - 1, H // 2})
-    Q, K, V, DO = (x.detach()[b].float().cpu().numpy().astype(np.float64) for x in (q, k, v, do))
-    OUT = out.detach()[b].cpu().numpy().astype(np.float64); LSE = lse[b].cpu().numpy().astype(np.float64)
-    DQ, DK, DV = (x.grad[b].float().cpu().numpy() for x in (q, k, v))
-    errs = {"out": 0.0, "lse": 0.0}
-    num = {"dq": 0.0, "dk": 0.0, "dv": 0.0}; den = {"dq": 0.0, "dk": 0.0, "dv": 0.0}
-    for h in heads:
-        for i in rows:
-            s = (K[:, h] @ Q[i, h]) * scale + bias_row(b, h, i)
-            mx = s.max(); p = np.exp(s - mx); l = p.sum()
-            o_i = (p @ V[:, h]) / l
-            errs["out"] = max(errs["out"], np.abs(OUT[i, h] - o_i).max())
-            errs["lse"] = max(errs["lse"], abs(LSE[h, i] - (mx + np.log(l))))
-            p = p / l
-            dp = V[:, h] @ DO[i, h]
-            ds = p * (dp - (p * dp).sum()) * scale
-            dq_i = ds @ K[:, h]
-            num["dq"] = max(num["dq"], np.abs(DQ[i, h] - dq_i).max()); den["dq"] = max(den["dq"], np.abs(dq_i).max())
-        delta = (OUT[:, h] * DO[:, h]).sum(axis=-1)
-        for j in cols:
-            s = (Q[:, h] @ K[j, h]) * scale + bias_col(b, h, j)
-            p = np.exp(s - LSE[h])
-            dv_j = p @ DO[:, h]
-            ds = p * (DO[:, h] @ V[j, h] - delta) * scale
-            dk_j = ds @ Q[:, h]
-            num["dv"] = max(num["dv"], np.abs(DV[j, h] - dv_j).max()); den["dv"] = max(den["dv"], np.abs(dv_j).max())
-            num["dk"] = max(num["dk"], np.abs(DK[j, h] - dk_j).max()); den["dk"] = max(den["dk"], np.abs(dk_j).max())
-    print(f"[parity] {name}: out {errs['out']:.2e} lse {errs['lse']:.2e} " +
-          " ".join(f"{kk} {num[kk] / den[kk]:.2e}" for kk in num), flush=True)
-    assert errs["out"] <= OUT_TOL and errs["lse"] <= LSE_TOL
-    for kk in num:
-        assert num[kk] / den[kk] <= GRAD_TOL, (kk, num[kk] / den[kk])
+    #   sum_j dv_j = sum_i do_i   (rows of P sum to one);   <q, dq> = <k, dk>   (both are sum_ij ds_ij s_ij / scale)
+    dv_sum, do_sum = v.grad.double().sum(dim=1), do.double().sum(dim=1)
+    inv1 = ((dv_sum - do_sum).abs().max() / do_sum.abs().max()).item()
+    qdq = (q.detach().double() * q.grad.double()).sum(dim=(1, 3))
+    kdk = (k.detach().double() * k.grad.double()).sum(dim=(1, 3))
+    inv2 = ((qdq - kdk).abs().max() / qdq.abs().max()).item()
+    assert inv1 <= GRAD_TOL and inv2 <= GRAD_TOL, (inv1, inv2)
+    L = S // n
+    edge = sorted({0, S - 1} | {min(max(c * L + d, 0), S - 1) for c in range(1, n) for d in (-1, 0, 1)})
+    worst = {"out": 0.0, "out_rel": 0.0, "lse": 0.0, "dq": 0.0, "dk": 0.0, "dv": 0.0, "ref_vs_oracle": 0.0}
+    for b in range(B):
+        for h in (sorted(heads) if heads is not None else range(H)):
+            Q, K, V, DO = (x.detach()[b, :, h].double() for x in (q, k, v, do))
+            r_out, r_lse, r_dq, r_dk, r_dv = _dense_reference_on_device(Q, K, V, DO, scale,
+                                                                       lambda i0, i1: bias_rows_t(b, h, i0, i1))
+            g_out, g_lse = out.detach()[b, :, h].double(), lse[b, h].double()
+            worst["out"] = max(worst["out"], (g_out - r_out).abs().max().item())
+            worst["out_rel"] = max(worst["out_rel"], ((g_out - r_out).abs().max() / r_out.abs().max()).item())
+            worst["lse"] = max(worst["lse"], (g_lse - r_lse).abs().max().item())
+            for nm, got, ref in (("dq", q.grad, r_dq), ("dk", k.grad, r_dk), ("dv", v.grad, r_dv)):
+                d = got[b, :, h].double() - ref
+                worst[nm] = max(worst[nm], (d.abs().max() / ref.abs().max()).item(),
+                                (d.norm() / ref.norm()).item())
+            # the oracle's formulas in numpy on sampled rows
+            rows = sorted(set(edge) | set(np.random.default_rng(1000 * b + h).integers(0, S, n_rows - len(edge)).tolist()))
+            Kn, Vn = K.cpu().numpy(), V.cpu().numpy()
+            Qn, DOn = Q[rows].cpu().numpy(), DO[rows].cpu().numpy()
+            t_out, t_lse, t_dq = r_out[rows].cpu().numpy(), r_lse[rows].cpu().numpy(), r_dq[rows].cpu().numpy()
+            sc_ = (Qn @ Kn.T) * scale + np.stack([bias_row_np(b, h, i) for i in rows])
+            mx = sc_.max(axis=1, keepdims=True)
+            pr = np.exp(sc_ - mx)
+            l_ = pr.sum(axis=1, keepdims=True)
+            pr /= l_
+            dp = DOn @ Vn.T
+            o_np = pr @ Vn
+            dq_np = (pr * (dp - (pr * dp).sum(axis=1, keepdims=True)) * scale) @ Kn
+            e = max(np.abs(t_out - o_np).max(), np.abs(t_lse - (mx + np.log(l_))[:, 0]).max(),
+                    (np.abs(t_dq - dq_np).max(axis=1) / (np.abs(dq_np).max(axis=1) + 1e-6)).max())
+            worst["ref_vs_oracle"] = max(worst["ref_vs_oracle"], float(e))
+    print(f"[parity] {name}: " + " ".join(f"{a} {b_:.2e}" for a, b_ in worst.items()) +
+          f" inv_dv {inv1:.2e} inv_qk {inv2:.2e}", flush=True)
+    assert worst["ref_vs_oracle"] <= 1e-9
+    assert worst["out"] <= OUT_TOL and worst["out_rel"] <= OUT_REL and worst["lse"] <= LSE_TOL, worst
+    for nm in ("dq", "dk", "dv"):
+        assert worst[nm] <= GRAD_TOL, worst
 
 
-def test_config2_full_size(device):
-    # B=2 H=16 D=128 S=8192 in 8 shards of 1024, causal with fully masked steps skipped
-    B, H, D, S, n = 2, 16, 128, 8192, 8
+def _causal_rows_t(device, S, window=None):
+    pos = torch.arange(S, device=device)
+
+    def rows(b, h, i0, i1):
+        rel = pos[i0:i1, None] - pos[None, :]
+        ok = rel >= 0 if window is None else (rel >= 0) & (rel < window)
+        return torch.where(ok, 0.0, -torch.inf).double()
+    return rows
+
+
+def _causal_row_np(S, window=None):
     pos = np.arange(S)
-    rows = [0, 1, 1023, 1024, 4095, 4096, 5000, S - 1]
-    cols = [0, 1023, 1024, 6000, S - 1]
-    _sampled_check(device, "C2", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
-                   lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf))
+    if window is None:
+        return lambda b, h, i: np.where(pos <= i, 0.0, -np.inf)
+    return lambda b, h, i: np.where((pos <= i) & (i - pos < window), 0.0, -np.inf)
 
 
-def test_config2_full_size_fused(device):
-    # the same workload with one launch per ring pass: small shards are where that pays
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_config2_full_size(device, impl):
+    # B=2 H=16 D=128 S=8192 in 8 shards of 1024, causal with fully masked steps skipped; every head,
+    # launch per step and launch per ring pass (small shards are where the latter pays)
     B, H, D, S, n = 2, 16, 128, 8192, 8
-    pos = np.arange(S)
-    rows = [0, 1, 1023, 1024, 4095, 4096, 5000, S - 1]
-    cols = [0, 1023, 1024, 6000, S - 1]
-    _sampled_check(device, "C2 fused", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
-                   lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf),
-                   impl="hip_fused")
+    _full_size_check(device, "C2", B, H, D, S, n, ra.causal_bias(), 1.0, _causal_rows_t(device, S),
+                     _causal_row_np(S), impl=impl, n_rows=64)
 
 
 def test_config3_full_size(device):
     # B=1 H=32 D=128 S=131072 in 8 shards of 16384, causal: the benchmark workload
     B, H, D, S, n = 1, 32, 128, 131072, 8
-    pos = np.arange(S)
-    rows = [0, 255, 16383, 16384, 70000, S - 1]
-    cols = [0, 16383, 16384, 100000, S - 1]
-    _sampled_check(device, "C3", B, H, D, S, n, ra.causal_bias(), 1.0, rows, cols,
-                   lambda b, h, i: np.where(pos <= i, 0.0, -np.inf), lambda b, h, j: np.where(pos >= j, 0.0, -np.inf))
+    _full_size_check(device, "C3", B, H, D, S, n, ra.causal_bias(), 1.0, _causal_rows_t(device, S),
+                     _causal_row_np(S), heads={0, 13, H - 1})
 
 
 def test_config4_full_size(device):
@@ -751,19 +930,20 @@ def test_config4_full_size(device):
     slopes = R.alibi_slopes(H)
     pos = np.arange(S)
     tseg = torch.from_numpy(seg).to(device)
-    rows = [0, 100, 8191, 8192, 20000, S - 1]
-    cols = [0, 8191, 8192, 30000, S - 1]
+    tpos = torch.arange(S, device=device)
+
+    def rows_t(b, h, i0, i1):
+        same = tseg[b, i0:i1, None] == tseg[b, None, :]
+        dist = (tpos[i0:i1, None] - tpos[None, :]).abs().double()
+        return torch.where(same, 0.0, -torch.inf).double() - float(slopes[h]) * dist
+
     brow = lambda b, h, i: np.where(seg[b] == seg[b, i], 0.0, -np.inf) - slopes[h] * np.abs(i - pos)
-    _sampled_check(device, "C4", B, H, D, S, n, ra.segment_bias() + ra.alibi_bias(slopes), 1.0, rows, cols,
-                   brow, brow, {"q_segment_ids": tseg}, {"kv_segment_ids": tseg})
+    _full_size_check(device, "C4", B, H, D, S, n, ra.segment_bias() + ra.alibi_bias(slopes), 1.0, rows_t, brow,
+                     {"q_segment_ids": tseg}, {"kv_segment_ids": tseg}, heads={0, 7, H - 1})
 
 
 def test_config5_full_size(device):
     # B=1 H=8 D=128 S=65536 in 8 shards of 8192, causal window 4096, N(0, 0.5^2)
     B, H, D, S, n, W = 1, 8, 128, 65536, 8, 4096
-    pos = np.arange(S)
-    rows = [0, 4095, 4096, 8191, 8192, 8193, 12287, 12288, 40000, S - 1]
-    cols = [0, 4096, 8191, 8192, 50000, S - 1]
-    _sampled_check(device, "C5", B, H, D, S, n, ra.sliding_window_bias(W), 0.5, rows, cols,
-                   lambda b, h, i: np.where((pos <= i) & (i - pos < W), 0.0, -np.inf),
-                   lambda b, h, j: np.where((pos >= j) & (pos - j < W), 0.0, -np.inf))
+    _full_size_check(device, "C5", B, H, D, S, n, ra.sliding_window_bias(W), 0.5, _causal_rows_t(device, S, W),
+                     _causal_row_np(S, W), heads={0, 3, H - 1})

@@ -73,8 +73,19 @@ def test_ring_plan_shards_and_offsets():
     pos = torch.cat([torch.arange(16) + 7 * i for i in range(4)])[None].repeat(2, 1)
     plan = rr._RingPlan(q, k, 4, ra.causal_bias(), {"q_positions": pos}, {})
     assert plan.q_off == [0, 7, 14, 21]
-    with pytest.raises(NotImplementedError):
-        rr._RingPlan(q, k, 4, ra.causal_bias(), {"q_positions": pos * 2}, {})
+    # any other positions are honoured through a dense block per ring step, built from the
+    # position arrays exactly like the reference's mask builder (ring.py:393-409)
+    plan = rr._RingPlan(q, k, 4, ra.causal_bias() + ra.segment_bias(),
+                        {"q_positions": pos * 2, "q_segment_ids": seg_q}, {"kv_segment_ids": seg_k})
+    assert plan.callable is not None and plan.fn is None
+    bb = plan.block_bias(1, 2)
+    assert tuple(bb.dense.shape) == (2, 1, 16, 8)
+    qp, kp = (pos * 2)[:, 16:32], torch.arange(32)[None].repeat(2, 1)[:, 16:24]
+    want = (kp[:, None, :] <= qp[:, :, None]) & (seg_q[:, 16:32, None] == seg_k[:, None, 16:24])
+    assert torch.equal(bb.dense[:, 0] == 0, want) and torch.equal(torch.isneginf(bb.dense[:, 0]), ~want)
+    # positions that differ across the batch take the same path
+    pos_b = torch.stack([torch.arange(64), torch.arange(64) + 3])
+    assert rr._RingPlan(q, k, 4, ra.causal_bias(), {"q_positions": pos_b}, {}).callable is not None
     with pytest.raises(ValueError):
         rr._RingPlan(q, k, 3, None, None, None)  # 64 % 3 != 0
     with pytest.raises(ValueError):
