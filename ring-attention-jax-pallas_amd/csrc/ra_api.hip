@@ -1,5 +1,6 @@
 // C ABI of the ring-attention block-step library: argument validation (host only, before
 // any HIP call) and dispatch to the gfx950 kernels.
+#include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -130,6 +131,10 @@ ra::BwdArgs to_bwd_args(const ra_bwd_step_params& p) {
   a.Lq = p.Lq;
   a.Lk = p.Lk;
   a.scale2 = p.sm_scale * kLog2eHost;
+  int e2 = 0;
+  const float mant = frexpf(a.scale2, &e2);  // scale2 = mant * 2^e2, mant in [0.5, 1)
+  a.scale_p2 = ldexpf(1.0f, e2 - 1);
+  a.scale_res = mant * 2.0f;
   a.sm_scale = p.sm_scale;
   a.bias = to_bias(p.bias);
   return a;

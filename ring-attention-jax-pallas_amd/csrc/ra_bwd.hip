@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
 
   __shared__ __attribute__((aligned(16))) char s_q[NB][TILE_BYTES];
   __shared__ __attribute__((aligned(16))) char s_do[NB][TILE_BYTES];
-  // per tile and row: -lse * log2(e) (-inf for a fully masked row), -delta, segment id, prefix flag
+  // per tile and row: -lse * log2(e) / scale_res (-inf for a fully masked row), -delta, segment id, prefix flag
   __shared__ __attribute__((aligned(16))) char s_stat[NB][STAT_BYTES];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
@@ -105,8 +105,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const bool wave_on = kw < a.Lk;
 
   // ---- resident key-side operands ----------------------------------------------------------
-  // K is scaled once, here, so that the score MFMAs deliver S * sm_scale * log2(e) directly;
-  // its rounding to bf16 perturbs a probability by a few 1e-3 relative, like the rounding of P.
+  // K is multiplied once, here, by the power of two below sm_scale * log2(e) - exact in bf16 - so
+  // that the score MFMAs deliver S * sm_scale * log2(e) / scale_res; the residual factor
+  // scale_res in [1, 2) is applied to the fp32 score in front of exp2, and everything that is
+  // added to a score tile (the row statistics, bias terms) is divided by it.  Folding the whole
+  // scale into the bf16 operand would perturb every probability by ~1e-3 relative (more with a
+  // wider score spread) and break the agreement with the forward pass's logsumexp.
   // They live in accumulation registers (the matrix unit reads its B operand from either file),
   // which leaves the vector registers to the score pipeline.
   u32x4 kfa[KS], vfa[KS];
@@ -120,7 +124,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     for (int s = 0; s < KS; ++s) {
       const bf16x8 kr = *(const bf16x8*)(kp + 16 * s);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) kf[s][e] = (bf16_t)((float)kr[e] * a.scale2);
+      for (int e = 0; e < 8; ++e) kf[s][e] = (bf16_t)((float)kr[e] * a.scale_p2);
       vf[s] = *(const bf16x8*)(vp + 16 * s);
     }
     if (GENERAL && (flags & RA_BIAS_SEGMENT)) k_seg = bs.kv_seg[b * bs.kv_seg_sb + ki];
@@ -143,7 +147,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "a"(b_acc));
   };
   float slope2 = 0.f;
-  if (GENERAL && (flags & RA_BIAS_ALIBI)) slope2 = bs.slopes[h] * kLog2e;
+  const float res = a.scale_res, inv_res = 1.0f / a.scale_res;
+  if (GENERAL && (flags & RA_BIAS_ALIBI)) slope2 = bs.slopes[h] * kLog2e * inv_res;
 
   f32x16 dk[DB], dv[DB];
   {
@@ -299,7 +304,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     st_src = st_class == 0 ? c0 : (st_class == 1 ? c1 : (st_class == 2 ? c2 : c3));
   }
   const unsigned st_dst = (unsigned)(st_class * (kQTile * 4) + st_row * 4);
-  const float st_mul = st_class == 0 ? -kLog2e : -1.0f;
+  const float st_mul = st_class == 0 ? -kLog2e * inv_res : -1.0f;
   const float st_fix = st_class == 0 ? RA_NEG_INF : 0.f;
   unsigned xr[3] = {0u, 0u, 0u};
   auto load_stat = [&](const char* p, unsigned& x) {
@@ -436,6 +441,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
+    tb.dense_mul = kLog2e * inv_res;
     tb.dense = nullptr;
     tb.dense_vs = 1;
     tb.var_limit = a.Lq - (qt0 + 4 * g);
@@ -533,7 +539,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
         float p[2], ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          p[e] = fast_exp2(SC[r + e]);
+          p[e] = fast_exp2(SC[r + e] * res);
           ds[e] = p[e] * PC[r + e];
         }
         pfw[r >> 3][(r & 7) >> 1] = pack2(p[0], p[1]);
@@ -659,7 +665,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       for (int e = 0; e < EPO; ++e) {
         const int r = op * EPO + e;
         if (r < 16) {
-          pe[r] = fast_exp2(SC[r]);
+          pe[r] = fast_exp2(SC[r] * res);
           asm volatile("" : "+v"(pe[r]));
         }
         if (r >= 1 && r <= 16) {
@@ -832,12 +838,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     const bf16_t* dp = a.dout.ptr + b * a.dout.sb + h * a.dout.sh + (long long)qi_c * a.dout.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
-      // Q is scaled once, here, so that the score MFMAs deliver S * sm_scale * log2(e) directly
-      // (its rounding to bf16 perturbs a probability by a few 1e-3 relative, like the rounding
-      // of P; dQ itself is built from the unscaled K)
+      // Q is multiplied once, here, by the power of two below sm_scale * log2(e) (exact in bf16);
+      // the residual factor scale_res in [1, 2) is applied to the fp32 score in front of exp2, as
+      // in the dK/dV kernel (dQ itself is built from the unscaled K)
       const bf16x8 qr = *(const bf16x8*)(qp + 16 * s);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) qf[s][e] = (bf16_t)((float)qr[e] * a.scale2);
+      for (int e = 0; e < 8; ++e) qf[s][e] = (bf16_t)((float)qr[e] * a.scale_p2);
       dof[s] = *(const bf16x8*)(dp + 16 * s);
     }
     if (TIGHT) {
@@ -865,7 +871,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   if (GENERAL) {
     if (flags & RA_BIAS_SEGMENT) q_seg = bs.q_seg[b * bs.q_seg_sb + qi_c];
     if (flags & RA_BIAS_PREFIX) q_pre = bs.q_pre[b * bs.q_pre_sb + qi_c];
-    if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e;
+    if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e / a.scale_res;
   }
   // ---- one pass of everything below per key/value shard ------------------------------------
   int kv_off = bs.kv_off;
@@ -1092,6 +1098,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
+    tb.dense_mul = kLog2e / a.scale_res;
     tb.dense = nullptr;
     tb.dense_vs = 1;
     const int var0 = kt0 + 4 * g;
@@ -1197,7 +1204,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         float ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          ds[e] = fast_exp2(SC[r + e] + neg_lse2) * (PC[r + e] - delta);
+          ds[e] = fast_exp2(fmaf(SC[r + e], a.scale_res, neg_lse2)) * (PC[r + e] - delta);
         }
         dsw[r >> 3][(r & 7) >> 1] = pack2(ds[0], ds[1]);
       }
@@ -1290,7 +1297,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       for (int e = 0; e < EPO; ++e) {
         const int r = slot * EPO + e;
         if (r >= 0 && r < 16) {
-          ev[r] = fast_exp2(SC[r]);
+          ev[r] = fast_exp2(SC[r] * a.scale_res);
           uv[r] = fmaf(PC[r], c_row, cd_row);
           asm volatile("" : "+v"(ev[r]), "+v"(uv[r]));  // pins the arithmetic between two MFMAs
         }

@@ -190,7 +190,8 @@ RA_DEV bf16x8 pack8(const f32x16& p, int base) {
 struct TileBias {
   int flags;     // terms that must be evaluated for this block
   int window;
-  float slope2;  // ALiBi slope * log2(e)
+  float slope2;  // ALiBi slope * log2(e), in the units of the score tile it is added to
+  float dense_mul;  // factor that takes a dense bias value (natural-log units) to those units
   int var_limit; // varying-side indices >= var_limit (relative to var0) are out of range
   const float* dense;   // dense bias element of (fixed index, var0); natural-log units
   long long dense_vs;   // its stride along the varying side (1 when the keys vary)
@@ -218,7 +219,7 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
       const int rel = QFIXED ? rel0 - off : rel0 + off;
       float x = t[r];
       if (tb.flags & RA_BIAS_ALIBI) x = fmaf(fabsf((float)rel), -tb.slope2, x);
-      if (DENSE) x = fmaf(dn[c], kLog2e, x);
+      if (DENSE) x = fmaf(dn[c], tb.dense_mul, x);
       bool msk = off >= tb.var_limit;
       if (tb.flags & RA_BIAS_CAUSAL) msk |= rel < 0;
       if (tb.flags & RA_BIAS_WINDOW) {

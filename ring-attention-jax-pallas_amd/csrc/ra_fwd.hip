@@ -429,6 +429,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
+    tb.dense_mul = kLog2e;
     tb.dense = nullptr;
     tb.dense_vs = 1;
     float mx = RA_NEG_INF;

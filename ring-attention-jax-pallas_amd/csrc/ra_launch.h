@@ -23,7 +23,9 @@ struct BwdArgs {
   float* dk;
   float* dv;
   int B, H, Lq, Lk;
-  float scale2;    // sm_scale * log2(e)
+  float scale2;    // sm_scale * log2(e) = scale_p2 * scale_res
+  float scale_p2;  // the power of two below scale2: folded into a bf16 operand without rounding
+  float scale_res; // scale2 / scale_p2 in [1, 2): applied to the fp32 scores
   float sm_scale;
   BiasArgs bias;
 };

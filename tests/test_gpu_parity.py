@@ -717,8 +717,9 @@ def test_seed0_ragged_sweep_cases(device, impl):
 @pytest.mark.parametrize("impl", ["hip", "hip_fused"])
 def test_seed0_ragged_sweep_cases_at_four_times_the_score_spread(device, impl):
     """The same cases with N(0, 2^2) inputs (what the hand-run sweep used): outside the amplitude
-    the absolute tolerances are stated for, so the output is held to a relative bound, and the
-    logsumexp and the gradients to theirs."""
+    the absolute tolerances are stated for, so the output is held to a relative bound; the
+    logsumexp and the gradients keep theirs (the backward kernels fold only a power of two of the
+    softmax scale into their bf16 operands, so a wider score spread costs them nothing)."""
     for case, kind, kw in _random_cases(0, max(_SEED0_RAGGED) + 1):
         if case not in _SEED0_RAGGED:
             continue
@@ -738,7 +739,7 @@ def test_seed0_ragged_sweep_cases_at_four_times_the_score_spread(device, impl):
         assert np.abs(lse - want_lse).max() <= LSE_TOL
         for got, ref, nm in zip(g, R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
             mx, fro = _rel(got, ref)
-            assert mx <= 3e-2 and fro <= 3e-2, (case, nm, mx, fro)
+            assert mx <= GRAD_TOL and fro <= GRAD_TOL, (case, nm, mx, fro)
 
 
 def test_delta_kernel(device):
