@@ -186,6 +186,42 @@ int ra_fwd_steps(const ra_fwd_step_params* steps, int32_t n_steps, void* stream)
 int ra_bwd_dq_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream);
 int ra_bwd_dkdv_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream);
 
+/* Several ring PASSES in one launch.  A pass is what ra_fwd_steps / ra_bwd_dq_steps /
+ * ra_bwd_dkdv_steps take: the steps of one resident shard's whole trip around the ring.  `steps`
+ * holds the passes one after another, pass p being the next steps_per_pass[p] blocks; the result
+ * is that of calling the *_steps entry point once per pass.  Passes are independent of each other
+ * (different query shards with their own carries or dq accumulators, or different key/value
+ * shards with their own dk / dv), so one grid runs them side by side: this is the loop nest of an
+ * emulated ring - all devices of ring.py:104-132 (forward) or ring.py:183-206 (backward) at once -
+ * for shards so small that one pass cannot fill the GPU.  Within a pass the blocks must agree as
+ * for *_steps; across passes they must share shape, strides, sm_scale and the bias terms (flags,
+ * window, id strides, slopes).  One launch covers at most 16 passes that draw from at most 16
+ * distinct travelling shards with at most 16 live steps each and no dense bias block; anything
+ * beyond that is issued pass by pass, with the same result. */
+int ra_fwd_passes(const ra_fwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes,
+                  void* stream);
+int ra_bwd_dq_passes(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes,
+                     void* stream);
+int ra_bwd_dkdv_passes(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes,
+                       void* stream);
+
+/* The elementwise entry points for the shards of n_passes passes in one launch: the fp32 arrays of
+ * the passes (carries, accumulators, lse, delta) lie one after another ([n_passes, B, H, L, ...]),
+ * pass p reads / writes its strided tensor at an offset of p * stride_pass elements.  With
+ * n_passes = 1 they are ra_fwd_finalize (ring.py:134-135,137), ra_bwd_delta
+ * (ring_kernel.py:387-409) and ra_bwd_finalize (ring.py:208-210). */
+int ra_fwd_finalize_passes(const float* o, const float* m, const float* l, void* out, int32_t out_dtype,
+                           int64_t out_stride_pass, int64_t out_stride_b, int64_t out_stride_h,
+                           int64_t out_stride_l, float* lse, int32_t n_passes, int32_t B, int32_t H,
+                           int32_t Lq, int32_t D, void* stream);
+int ra_bwd_delta_passes(const void* out, int32_t out_dtype, int64_t out_stride_pass, int64_t out_stride_b,
+                        int64_t out_stride_h, int64_t out_stride_l, const ra_tensor* dout,
+                        int64_t dout_stride_pass, float* delta, int32_t n_passes, int32_t B, int32_t H,
+                        int32_t Lq, int32_t D, void* stream);
+int ra_bwd_finalize_passes(const float* acc, void* out, int64_t out_stride_pass, int64_t out_stride_b,
+                           int64_t out_stride_h, int64_t out_stride_l, int32_t n_passes, int32_t B,
+                           int32_t H, int32_t L, int32_t D, void* stream);
+
 /* Host-only, pure: 1 if every score of the (query shard, key/value shard) pair is masked
  * by the positional terms of `bias` (CAUSAL / WINDOW), so that the whole ring step is an
  * identity on the carry and may be skipped; 0 otherwise.  The reference runs such steps and

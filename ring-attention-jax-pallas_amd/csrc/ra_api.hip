@@ -5,6 +5,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
+#include <vector>
+
 #include "ra_launch.h"
 
 namespace {
@@ -168,21 +171,291 @@ bool same_kv_side(const ra_bias& x, const ra_bias& y) {
          x.dense_stride_h == y.dense_stride_h && x.dense_stride_q == y.dense_stride_q;
 }
 
-void add_kv_shard(ra::KvShardList& sl, const ra_tensor& k, const ra_tensor& v, const ra_bias& b) {
-  const int i = sl.n++;
-  sl.kv_off[i] = (int)b.kv_offset;
-  sl.k[i] = (const ra::bf16_t*)k.ptr;
-  sl.v[i] = (const ra::bf16_t*)v.ptr;
-  sl.kv_seg[i] = b.kv_segment_ids;
-  sl.kv_pre[i] = b.kv_prefix;
-  sl.dense[i] = b.dense_bias;
+// ---- launches that walk several shards, and several ring passes per launch ------------------------
+// The travelling side of a step, as the shared table of a ring launch holds it.
+struct KvEntry {
+  const void* k; const void* v; int64_t off; const int32_t* seg; const int32_t* pre; const float* dense;
+  bool operator==(const KvEntry& o) const {
+    return k == o.k && v == o.v && off == o.off && seg == o.seg && pre == o.pre && dense == o.dense;
+  }
+};
+struct QEntry {
+  const void* q; const void* dout; const float* lse; const float* delta; int64_t off; const int32_t* seg;
+  const int32_t* pre; const float* dense;
+  bool operator==(const QEntry& o) const {
+    return q == o.q && dout == o.dout && lse == o.lse && delta == o.delta && off == o.off && seg == o.seg &&
+           pre == o.pre && dense == o.dense;
+  }
+};
+KvEntry kv_entry(const ra_tensor& k, const ra_tensor& v, const ra_bias& b) {
+  return KvEntry{k.ptr, v.ptr, b.kv_offset, b.kv_segment_ids, b.kv_prefix, b.dense_bias};
+}
+QEntry q_entry(const ra_bwd_step_params& p) {
+  return QEntry{p.q.ptr, p.dout.ptr, p.lse, p.delta, p.bias.q_offset, p.bias.q_segment_ids, p.bias.q_prefix,
+                p.bias.dense_bias};
+}
+void put(ra::KvShardList& t, int i, const KvEntry& e) {
+  t.kv_off[i] = (int)e.off;
+  t.k[i] = (const ra::bf16_t*)e.k;
+  t.v[i] = (const ra::bf16_t*)e.v;
+  t.kv_seg[i] = e.seg;
+  t.kv_pre[i] = e.pre;
+  t.dense[i] = e.dense;
+}
+void put(ra::QShardList& t, int i, const QEntry& e) {
+  t.q_off[i] = (int)e.off;
+  t.q[i] = (const ra::bf16_t*)e.q;
+  t.dout[i] = (const ra::bf16_t*)e.dout;
+  t.lse[i] = e.lse;
+  t.delta[i] = e.delta;
+  t.q_seg[i] = e.seg;
+  t.q_pre[i] = e.pre;
+  t.dense[i] = e.dense;
+}
+
+// Plans the launches of `n_passes` ring passes whose live steps (entries of the travelling side)
+// are entries[first[p] .. first[p + 1]).  If every pass has at most kMaxShards live steps, there
+// are at most kMaxPasses passes and the passes draw from at most kMaxShards distinct shards, ONE
+// launch covers them all (heaviest pass first: it is dispatched first); otherwise every pass gets
+// its own launches of at most kMaxShards steps each.  Ring is KvRing or QRing, `set_pass(ring,
+// slot, p)` fills the resident side of pass p into slot `slot`, `launch(ring)` enqueues.
+template <typename Ring, typename Table, typename Entry, typename SetPass, typename Launch>
+int run_passes(Table Ring::*table, const std::vector<Entry>& entries, const std::vector<int>& first, int n_passes,
+               SetPass set_pass, Launch launch) {
+  std::vector<Entry> distinct;
+  std::vector<int> index(entries.size());
+  bool one_launch = n_passes <= ra::kMaxPasses;
+  for (size_t i = 0; i < entries.size() && one_launch; ++i) {
+    size_t j = 0;
+    while (j < distinct.size() && !(distinct[j] == entries[i])) ++j;
+    if (j == distinct.size()) {
+      if ((int)distinct.size() == ra::kMaxShards) one_launch = false;
+      else distinct.push_back(entries[i]);
+    }
+    index[i] = (int)j;
+  }
+  for (int p = 0; p < n_passes && one_launch; ++p) one_launch = first[p + 1] - first[p] <= ra::kMaxShards;
+  Ring ring;
+  memset(&ring, 0, sizeof(ring));
+  if (one_launch) {
+    for (size_t j = 0; j < distinct.size(); ++j) put(ring.*table, (int)j, distinct[j]);
+    (ring.*table).n = (int)distinct.size();
+    std::vector<int> by_weight;
+    for (int p = 0; p < n_passes; ++p)
+      if (first[p + 1] > first[p]) by_weight.push_back(p);
+    std::stable_sort(by_weight.begin(), by_weight.end(),
+                     [&](int x, int y) { return first[x + 1] - first[x] > first[y + 1] - first[y]; });
+    if (by_weight.empty()) return RA_OK;
+    ring.n_pass = (int)by_weight.size();
+    for (int slot = 0; slot < ring.n_pass; ++slot) {
+      const int p = by_weight[slot];
+      ring.count[slot] = (unsigned char)(first[p + 1] - first[p]);
+      for (int i = first[p]; i < first[p + 1]; ++i) ring.order[slot][i - first[p]] = (unsigned char)index[i];
+      set_pass(ring, slot, p);
+    }
+    return launch(ring);
+  }
+  for (int p = 0; p < n_passes; ++p) {
+    for (int i0 = first[p]; i0 < first[p + 1]; i0 += ra::kMaxShards) {
+      const int cnt = std::min(ra::kMaxShards, first[p + 1] - i0);
+      memset(&ring, 0, sizeof(ring));
+      for (int i = 0; i < cnt; ++i) {
+        put(ring.*table, i, entries[i0 + i]);
+        ring.order[0][i] = (unsigned char)i;
+      }
+      (ring.*table).n = cnt;
+      ring.n_pass = 1;
+      ring.count[0] = (unsigned char)cnt;
+      set_pass(ring, 0, p);
+      int rc = launch(ring);
+      if (rc) return rc;
+    }
+  }
+  return RA_OK;
+}
+
+// the fields of a bias description that every step of a launch must share
+bool same_bias_shape(const ra_bias& x, const ra_bias& y) {
+  return x.flags == y.flags && x.window == y.window && x.q_segment_stride_b == y.q_segment_stride_b &&
+         x.kv_segment_stride_b == y.kv_segment_stride_b && x.q_prefix_stride_b == y.q_prefix_stride_b &&
+         x.kv_prefix_stride_b == y.kv_prefix_stride_b && x.alibi_slopes == y.alibi_slopes &&
+         x.dense_stride_b == y.dense_stride_b && x.dense_stride_h == y.dense_stride_h &&
+         x.dense_stride_q == y.dense_stride_q;
+}
+
+int check_pass_counts(const int32_t* steps_per_pass, int32_t n_passes, std::vector<int>& first) {
+  if (n_passes < 0) return fail(RA_ERR_SHAPE, "n_passes is negative");
+  if (n_passes > 0 && !steps_per_pass) return fail(RA_ERR_NULL, "steps_per_pass is NULL");
+  first.assign(1, 0);
+  for (int p = 0; p < n_passes; ++p) {
+    if (steps_per_pass[p] < 0) return fail(RA_ERR_SHAPE, "steps_per_pass[%d] is negative", p);
+    first.push_back(first.back() + steps_per_pass[p]);
+  }
+  return RA_OK;
+}
+
+int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream) {
+  const int total = first.back();
+  if (total == 0) return RA_OK;
+  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
+  const ra_fwd_step_params& f = steps[0];
+  for (int p = 0; p < n_passes; ++p) {
+    for (int i = first[p]; i < first[p + 1]; ++i) {
+      const ra_fwd_step_params& s = steps[i];
+      const ra_fwd_step_params& h = steps[first[p]];  // head of the pass
+      int rc = ra_fwd_step_check(&s);
+      if (rc) return rc;
+      const bool shape = s.B == f.B && s.H == f.H && s.Lq == f.Lq && s.Lk == f.Lk && s.D == f.D &&
+                         s.sm_scale == f.sm_scale && same_strides(s.q, f.q) && same_strides(s.k, f.k) &&
+                         same_strides(s.v, f.v) && same_bias_shape(s.bias, f.bias);
+      const bool pass = !memcmp(&s.q, &h.q, sizeof(ra_tensor)) && s.o == h.o && s.m == h.m && s.l == h.l &&
+                        same_q_side(s.bias, h.bias);
+      if (!shape || !pass)
+        return fail(RA_ERR_SHAPE, "steps[%d] differs from the first step of its pass in more than its key/value shard "
+                                  "(k.ptr, v.ptr, kv_offset, kv_segment_ids, kv_prefix, dense_bias), or from "
+                                  "steps[0] in shape, strides or bias terms", i);
+    }
+  }
+  ra::FwdArgs a;
+  a.q = to_arg(f.q);
+  a.k = to_arg(f.k);
+  a.v = to_arg(f.v);
+  a.o = f.o;
+  a.m = f.m;
+  a.l = f.l;
+  a.B = f.B;
+  a.H = f.H;
+  a.Lq = f.Lq;
+  a.Lk = f.Lk;
+  a.scale2 = f.sm_scale * kLog2eHost;
+  a.bias = to_bias(f.bias);
+  // live steps only: a masked step is an identity on the carry
+  std::vector<KvEntry> entries;
+  std::vector<int> live_first(1, 0), head(n_passes, 0);
+  for (int p = 0; p < n_passes; ++p) {
+    head[p] = first[p];
+    for (int i = first[p]; i < first[p + 1]; ++i)
+      if (!ra_step_is_skippable(&steps[i].bias, steps[i].Lq, steps[i].Lk))
+        entries.push_back(kv_entry(steps[i].k, steps[i].v, steps[i].bias));
+    live_first.push_back((int)entries.size());
+  }
+  auto set_pass = [&](ra::KvRing& r, int slot, int p) {
+    const ra_fwd_step_params& h = steps[head[p]];
+    r.q_off[slot] = (int)h.bias.q_offset;
+    r.q[slot] = (const ra::bf16_t*)h.q.ptr;
+    r.x0[slot] = h.o;
+    r.x1[slot] = h.m;
+    r.x2[slot] = h.l;
+    r.q_seg[slot] = h.bias.q_segment_ids;
+    r.q_pre[slot] = h.bias.q_prefix;
+  };
+  auto launch = [&](const ra::KvRing& r) -> int {
+    hipError_t e = ra::launch_fwd_steps(a, r, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
+    return e == hipSuccess ? RA_OK : hip_fail(e, "forward ring launch");
+  };
+  return run_passes<ra::KvRing>(&ra::KvRing::kv, entries, live_first, n_passes, set_pass, launch);
+}
+
+int bwd_dq_passes(const ra_bwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream) {
+  const int total = first.back();
+  if (total == 0) return RA_OK;
+  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
+  const ra_bwd_step_params& f = steps[0];
+  for (int p = 0; p < n_passes; ++p) {
+    for (int i = first[p]; i < first[p + 1]; ++i) {
+      const ra_bwd_step_params& s = steps[i];
+      const ra_bwd_step_params& h = steps[first[p]];
+      int rc = ra_bwd_step_check(&s);
+      if (rc) return rc;
+      const bool shape = same_dims(s, f) && same_strides(s.q, f.q) && same_strides(s.dout, f.dout) &&
+                         same_strides(s.k, f.k) && same_strides(s.v, f.v) && same_bias_shape(s.bias, f.bias);
+      const bool pass = !memcmp(&s.q, &h.q, sizeof(ra_tensor)) && !memcmp(&s.dout, &h.dout, sizeof(ra_tensor)) &&
+                        s.lse == h.lse && s.delta == h.delta && s.dq == h.dq && same_q_side(s.bias, h.bias);
+      if (!shape || !pass)
+        return fail(RA_ERR_SHAPE, "steps[%d] differs from the first step of its pass in more than its key/value shard "
+                                  "(k.ptr, v.ptr, dk, dv, kv_offset, kv_segment_ids, kv_prefix, dense_bias), or from "
+                                  "steps[0] in shape, strides or bias terms", i);
+    }
+  }
+  const ra::BwdArgs a = to_bwd_args(f);
+  std::vector<KvEntry> entries;
+  std::vector<int> live_first(1, 0);
+  for (int p = 0; p < n_passes; ++p) {
+    for (int i = first[p]; i < first[p + 1]; ++i)
+      if (!ra_step_is_skippable(&steps[i].bias, steps[i].Lq, steps[i].Lk))  // contributes nothing
+        entries.push_back(kv_entry(steps[i].k, steps[i].v, steps[i].bias));
+    live_first.push_back((int)entries.size());
+  }
+  auto set_pass = [&](ra::KvRing& r, int slot, int p) {
+    const ra_bwd_step_params& h = steps[first[p]];
+    r.q_off[slot] = (int)h.bias.q_offset;
+    r.q[slot] = (const ra::bf16_t*)h.q.ptr;
+    r.dout[slot] = (const ra::bf16_t*)h.dout.ptr;
+    r.x0[slot] = h.dq;
+    r.x1[slot] = const_cast<float*>(h.lse);
+    r.x2[slot] = const_cast<float*>(h.delta);
+    r.q_seg[slot] = h.bias.q_segment_ids;
+    r.q_pre[slot] = h.bias.q_prefix;
+  };
+  auto launch = [&](const ra::KvRing& r) -> int {
+    hipError_t e = ra::launch_bwd_dq_steps(a, r, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
+    return e == hipSuccess ? RA_OK : hip_fail(e, "dQ ring launch");
+  };
+  return run_passes<ra::KvRing>(&ra::KvRing::kv, entries, live_first, n_passes, set_pass, launch);
+}
+
+int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream) {
+  const int total = first.back();
+  if (total == 0) return RA_OK;
+  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
+  const ra_bwd_step_params& f = steps[0];
+  for (int p = 0; p < n_passes; ++p) {
+    for (int i = first[p]; i < first[p + 1]; ++i) {
+      const ra_bwd_step_params& s = steps[i];
+      const ra_bwd_step_params& h = steps[first[p]];
+      int rc = ra_bwd_step_check(&s);
+      if (rc) return rc;
+      const bool shape = same_dims(s, f) && same_strides(s.q, f.q) && same_strides(s.dout, f.dout) &&
+                         same_strides(s.k, f.k) && same_strides(s.v, f.v) && same_bias_shape(s.bias, f.bias);
+      const bool pass = !memcmp(&s.k, &h.k, sizeof(ra_tensor)) && !memcmp(&s.v, &h.v, sizeof(ra_tensor)) &&
+                        s.dk == h.dk && s.dv == h.dv && same_kv_side(s.bias, h.bias);
+      if (!shape || !pass)
+        return fail(RA_ERR_SHAPE, "steps[%d] differs from the first step of its pass in more than its query shard (q.ptr, "
+                                  "dout.ptr, lse, delta, dq, q_offset, q_segment_ids, q_prefix, dense_bias), or from "
+                                  "steps[0] in shape, strides or bias terms", i);
+    }
+  }
+  const ra::BwdArgs a = to_bwd_args(f);
+  std::vector<QEntry> entries;
+  std::vector<int> live_first(1, 0);
+  for (int p = 0; p < n_passes; ++p) {
+    for (int i = first[p]; i < first[p + 1]; ++i)
+      if (!ra_step_is_skippable(&steps[i].bias, steps[i].Lq, steps[i].Lk))  // contributes nothing
+        entries.push_back(q_entry(steps[i]));
+    live_first.push_back((int)entries.size());
+  }
+  auto set_pass = [&](ra::QRing& r, int slot, int p) {
+    const ra_bwd_step_params& h = steps[first[p]];
+    r.kv_off[slot] = (int)h.bias.kv_offset;
+    r.k[slot] = (const ra::bf16_t*)h.k.ptr;
+    r.v[slot] = (const ra::bf16_t*)h.v.ptr;
+    r.dk[slot] = h.dk;
+    r.dv[slot] = h.dv;
+    r.kv_seg[slot] = h.bias.kv_segment_ids;
+    r.kv_pre[slot] = h.bias.kv_prefix;
+  };
+  auto launch = [&](const ra::QRing& r) -> int {
+    hipError_t e = ra::launch_bwd_dkdv_steps(a, r, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
+    return e == hipSuccess ? RA_OK : hip_fail(e, "dK/dV ring launch");
+  };
+  return run_passes<ra::QRing>(&ra::QRing::q, entries, live_first, n_passes, set_pass, launch);
 }
 
 }  // namespace
 
 extern "C" {
 
-int ra_version(void) { return 1003; }
+int ra_version(void) { return 1004; }
 
 const char* ra_last_error(void) { return g_err; }
 
@@ -261,89 +534,71 @@ int ra_fwd_step(const ra_fwd_step_params* p, void* stream) {
 
 int ra_fwd_steps(const ra_fwd_step_params* steps, int32_t n_steps, void* stream) {
   if (n_steps < 0) return fail(RA_ERR_SHAPE, "n_steps is negative");
-  if (n_steps == 0) return RA_OK;
-  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
-  const ra_fwd_step_params& f = steps[0];
-  for (int i = 0; i < n_steps; ++i) {
-    const ra_fwd_step_params& p = steps[i];
-    int rc = ra_fwd_step_check(&p);
-    if (rc) return rc;
-    const bool same =
-        p.B == f.B && p.H == f.H && p.Lq == f.Lq && p.Lk == f.Lk && p.D == f.D && p.sm_scale == f.sm_scale &&
-        !memcmp(&p.q, &f.q, sizeof(ra_tensor)) && p.o == f.o && p.m == f.m && p.l == f.l &&
-        same_strides(p.k, f.k) && same_strides(p.v, f.v) && same_q_side(p.bias, f.bias);
-    if (!same)
-      return fail(RA_ERR_SHAPE, "steps[%d] differs from steps[0] in more than its key/value shard "
-                                "(k.ptr, v.ptr, kv_offset, kv_segment_ids, kv_prefix, dense_bias)", i);
-  }
-  ra::FwdArgs a;
-  a.q = to_arg(f.q);
-  a.k = to_arg(f.k);
-  a.v = to_arg(f.v);
-  a.o = f.o;
-  a.m = f.m;
-  a.l = f.l;
-  a.B = f.B;
-  a.H = f.H;
-  a.Lq = f.Lq;
-  a.Lk = f.Lk;
-  a.scale2 = f.sm_scale * kLog2eHost;
-  a.bias = to_bias(f.bias);
-  ra::KvShardList sl;
-  memset(&sl, 0, sizeof(sl));
-  auto flush = [&]() -> int {
-    if (sl.n == 0) return RA_OK;
-    hipError_t e = ra::launch_fwd_steps(a, sl, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
-    sl.n = 0;
-    return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_steps launch");
-  };
-  for (int i = 0; i < n_steps; ++i) {
-    const ra_fwd_step_params& p = steps[i];
-    if (ra_step_is_skippable(&p.bias, p.Lq, p.Lk)) continue;  // identity on the carry
-    add_kv_shard(sl, p.k, p.v, p.bias);
-    if (sl.n == ra::kMaxShards) {
-      int rc = flush();
-      if (rc) return rc;
-    }
-  }
-  return flush();
+  return fwd_passes(steps, std::vector<int>{0, n_steps}, 1, stream);
 }
 
-int ra_fwd_finalize(const float* o, const float* m, const float* l, void* out, int32_t out_dtype,
-                    int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l, float* lse,
-                    int32_t B, int32_t H, int32_t Lq, int32_t D, void* stream) {
+int ra_fwd_passes(const ra_fwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* stream) {
+  std::vector<int> first;
+  int rc = check_pass_counts(steps_per_pass, n_passes, first);
+  return rc ? rc : fwd_passes(steps, first, n_passes, stream);
+}
+
+int ra_fwd_finalize_passes(const float* o, const float* m, const float* l, void* out, int32_t out_dtype,
+                           int64_t out_stride_pass, int64_t out_stride_b, int64_t out_stride_h,
+                           int64_t out_stride_l, float* lse, int32_t n_passes, int32_t B, int32_t H, int32_t Lq,
+                           int32_t D, void* stream) {
   if (!o || !m || !l || !out || !lse) return fail(RA_ERR_NULL, "ra_fwd_finalize: NULL pointer");
+  if (n_passes <= 0 || n_passes > (1 << 16)) return fail(RA_ERR_SHAPE, "n_passes must lie in [1, 65536]");
   int rc = check_dims(B, H, Lq, 1, D);
   if (rc) return rc;
+  if ((int64_t)n_passes * B * H > (1 << 20)) return fail(RA_ERR_SHAPE, "n_passes*B*H too large");
   if (out_dtype != RA_DTYPE_BF16 && out_dtype != RA_DTYPE_F32)
     return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
-  if ((out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
+  if ((out_stride_pass % 4) || (out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
     return fail(RA_ERR_ALIGN, "out strides must be multiples of 4 elements");
   // the kernel stores four elements at a time: 8 bytes of bf16 or 16 bytes of fp32
   if (reinterpret_cast<uintptr_t>(out) % (out_dtype == RA_DTYPE_F32 ? 16u : 8u))
     return fail(RA_ERR_ALIGN, "out must be aligned to four elements (%d bytes)", out_dtype == RA_DTYPE_F32 ? 16 : 8);
   if (!aligned16(o)) return fail(RA_ERR_ALIGN, "o is not 16-byte aligned");
-  hipError_t e = ra::launch_fwd_finalize(o, m, l, out, out_dtype == RA_DTYPE_F32, out_stride_b,
-                                         out_stride_h, out_stride_l, lse, B, H, Lq, D,
+  hipError_t e = ra::launch_fwd_finalize(o, m, l, out, out_dtype == RA_DTYPE_F32, out_stride_pass, out_stride_b,
+                                         out_stride_h, out_stride_l, lse, n_passes, B, H, Lq, D,
                                          (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_finalize launch");
+}
+
+int ra_fwd_finalize(const float* o, const float* m, const float* l, void* out, int32_t out_dtype,
+                    int64_t out_stride_b, int64_t out_stride_h, int64_t out_stride_l, float* lse,
+                    int32_t B, int32_t H, int32_t Lq, int32_t D, void* stream) {
+  return ra_fwd_finalize_passes(o, m, l, out, out_dtype, 0, out_stride_b, out_stride_h, out_stride_l, lse, 1, B, H,
+                                Lq, D, stream);
+}
+
+int ra_bwd_delta_passes(const void* out, int32_t out_dtype, int64_t out_stride_pass, int64_t out_stride_b,
+                        int64_t out_stride_h, int64_t out_stride_l, const ra_tensor* dout,
+                        int64_t dout_stride_pass, float* delta, int32_t n_passes, int32_t B, int32_t H,
+                        int32_t Lq, int32_t D, void* stream) {
+  if (!out || !dout || !delta) return fail(RA_ERR_NULL, "ra_bwd_delta: NULL pointer");
+  if (n_passes <= 0 || n_passes > (1 << 16)) return fail(RA_ERR_SHAPE, "n_passes must lie in [1, 65536]");
+  int rc = check_dims(B, H, Lq, 1, D);
+  if (rc) return rc;
+  if ((int64_t)n_passes * B * H > (1 << 20)) return fail(RA_ERR_SHAPE, "n_passes*B*H too large");
+  if ((rc = check_tensor("dout", *dout))) return rc;
+  if (out_dtype != RA_DTYPE_BF16 && out_dtype != RA_DTYPE_F32)
+    return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
+  if (!aligned16(out) || (out_stride_pass % 8) || (out_stride_b % 8) || (out_stride_h % 8) || (out_stride_l % 8) ||
+      (dout_stride_pass % 8))
+    return fail(RA_ERR_ALIGN, "out must be 16-byte aligned with strides that are multiples of 8");
+  hipError_t e = ra::launch_bwd_delta(out, out_dtype == RA_DTYPE_F32, out_stride_pass, out_stride_b, out_stride_h,
+                                      out_stride_l, to_arg(*dout), dout_stride_pass, delta, n_passes, B, H, Lq, D,
+                                      (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_delta launch");
 }
 
 int ra_bwd_delta(const void* out, int32_t out_dtype, int64_t out_stride_b, int64_t out_stride_h,
                  int64_t out_stride_l, const ra_tensor* dout, float* delta, int32_t B, int32_t H,
                  int32_t Lq, int32_t D, void* stream) {
-  if (!out || !dout || !delta) return fail(RA_ERR_NULL, "ra_bwd_delta: NULL pointer");
-  int rc = check_dims(B, H, Lq, 1, D);
-  if (rc) return rc;
-  if ((rc = check_tensor("dout", *dout))) return rc;
-  if (out_dtype != RA_DTYPE_BF16 && out_dtype != RA_DTYPE_F32)
-    return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
-  if (!aligned16(out) || (out_stride_b % 8) || (out_stride_h % 8) || (out_stride_l % 8))
-    return fail(RA_ERR_ALIGN, "out must be 16-byte aligned with strides that are multiples of 8");
-  hipError_t e = ra::launch_bwd_delta(out, out_dtype == RA_DTYPE_F32, out_stride_b, out_stride_h,
-                                      out_stride_l, to_arg(*dout), delta, B, H, Lq, D,
-                                      (hipStream_t)stream);
-  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_delta launch");
+  return ra_bwd_delta_passes(out, out_dtype, 0, out_stride_b, out_stride_h, out_stride_l, dout, 0, delta, 1, B, H, Lq,
+                             D, stream);
 }
 
 int ra_bwd_step(const ra_bwd_step_params* p, void* stream) { return ra_bwd_step_parts(p, 3, stream); }
@@ -360,100 +615,49 @@ int ra_bwd_step_parts(const ra_bwd_step_params* p, int32_t parts, void* stream) 
 
 int ra_bwd_dq_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream) {
   if (n_steps < 0) return fail(RA_ERR_SHAPE, "n_steps is negative");
-  if (n_steps == 0) return RA_OK;
-  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
-  const ra_bwd_step_params& f = steps[0];
-  for (int i = 0; i < n_steps; ++i) {
-    const ra_bwd_step_params& p = steps[i];
-    int rc = ra_bwd_step_check(&p);
-    if (rc) return rc;
-    const bool same = same_dims(p, f) && !memcmp(&p.q, &f.q, sizeof(ra_tensor)) &&
-                      !memcmp(&p.dout, &f.dout, sizeof(ra_tensor)) && p.lse == f.lse && p.delta == f.delta &&
-                      p.dq == f.dq && same_strides(p.k, f.k) && same_strides(p.v, f.v) &&
-                      same_q_side(p.bias, f.bias);
-    if (!same)
-      return fail(RA_ERR_SHAPE, "steps[%d] differs from steps[0] in more than its key/value shard "
-                                "(k.ptr, v.ptr, dk, dv, kv_offset, kv_segment_ids, kv_prefix, dense_bias)", i);
-  }
-  const ra::BwdArgs a = to_bwd_args(f);
-  ra::KvShardList sl;
-  memset(&sl, 0, sizeof(sl));
-  auto flush = [&]() -> int {
-    if (sl.n == 0) return RA_OK;
-    hipError_t e = ra::launch_bwd_dq_steps(a, sl, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
-    sl.n = 0;
-    return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_dq_steps launch");
-  };
-  for (int i = 0; i < n_steps; ++i) {
-    const ra_bwd_step_params& p = steps[i];
-    if (ra_step_is_skippable(&p.bias, p.Lq, p.Lk)) continue;  // contributes nothing
-    add_kv_shard(sl, p.k, p.v, p.bias);
-    if (sl.n == ra::kMaxShards) {
-      int rc = flush();
-      if (rc) return rc;
-    }
-  }
-  return flush();
+  return bwd_dq_passes(steps, std::vector<int>{0, n_steps}, 1, stream);
 }
 
 int ra_bwd_dkdv_steps(const ra_bwd_step_params* steps, int32_t n_steps, void* stream) {
   if (n_steps < 0) return fail(RA_ERR_SHAPE, "n_steps is negative");
-  if (n_steps == 0) return RA_OK;
-  if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
-  const ra_bwd_step_params& f = steps[0];
-  for (int i = 0; i < n_steps; ++i) {
-    const ra_bwd_step_params& p = steps[i];
-    int rc = ra_bwd_step_check(&p);
-    if (rc) return rc;
-    const bool same = same_dims(p, f) && !memcmp(&p.k, &f.k, sizeof(ra_tensor)) &&
-                      !memcmp(&p.v, &f.v, sizeof(ra_tensor)) && p.dk == f.dk && p.dv == f.dv &&
-                      same_strides(p.q, f.q) && same_strides(p.dout, f.dout) && same_kv_side(p.bias, f.bias);
-    if (!same)
-      return fail(RA_ERR_SHAPE, "steps[%d] differs from steps[0] in more than its query shard (q.ptr, "
-                                "dout.ptr, lse, delta, dq, q_offset, q_segment_ids, q_prefix, dense_bias)", i);
-  }
-  const ra::BwdArgs a = to_bwd_args(f);
-  ra::QShardList sl;
-  memset(&sl, 0, sizeof(sl));
-  auto flush = [&]() -> int {
-    if (sl.n == 0) return RA_OK;
-    hipError_t e = ra::launch_bwd_dkdv_steps(a, sl, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
-    sl.n = 0;
-    return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_dkdv_steps launch");
-  };
-  for (int i = 0; i < n_steps; ++i) {
-    const ra_bwd_step_params& p = steps[i];
-    if (ra_step_is_skippable(&p.bias, p.Lq, p.Lk)) continue;  // contributes nothing
-    const int j = sl.n++;
-    sl.q_off[j] = (int)p.bias.q_offset;
-    sl.q[j] = (const ra::bf16_t*)p.q.ptr;
-    sl.dout[j] = (const ra::bf16_t*)p.dout.ptr;
-    sl.lse[j] = p.lse;
-    sl.delta[j] = p.delta;
-    sl.q_seg[j] = p.bias.q_segment_ids;
-    sl.q_pre[j] = p.bias.q_prefix;
-    sl.dense[j] = p.bias.dense_bias;
-    if (sl.n == ra::kMaxShards) {
-      int rc = flush();
-      if (rc) return rc;
-    }
-  }
-  return flush();
+  return bwd_dkdv_passes(steps, std::vector<int>{0, n_steps}, 1, stream);
 }
 
-int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t out_stride_h,
-                    int64_t out_stride_l, int32_t B, int32_t H, int32_t L, int32_t D, void* stream) {
+int ra_bwd_dq_passes(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes,
+                     void* stream) {
+  std::vector<int> first;
+  int rc = check_pass_counts(steps_per_pass, n_passes, first);
+  return rc ? rc : bwd_dq_passes(steps, first, n_passes, stream);
+}
+
+int ra_bwd_dkdv_passes(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes,
+                       void* stream) {
+  std::vector<int> first;
+  int rc = check_pass_counts(steps_per_pass, n_passes, first);
+  return rc ? rc : bwd_dkdv_passes(steps, first, n_passes, stream);
+}
+
+int ra_bwd_finalize_passes(const float* acc, void* out, int64_t out_stride_pass, int64_t out_stride_b,
+                           int64_t out_stride_h, int64_t out_stride_l, int32_t n_passes, int32_t B, int32_t H,
+                           int32_t L, int32_t D, void* stream) {
   if (!acc || !out) return fail(RA_ERR_NULL, "ra_bwd_finalize: NULL pointer");
+  if (n_passes <= 0 || n_passes > (1 << 16)) return fail(RA_ERR_SHAPE, "n_passes must lie in [1, 65536]");
   int rc = check_dims(B, H, L, 1, D);
   if (rc) return rc;
-  if ((out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
+  if ((int64_t)n_passes * B * H > (1 << 20)) return fail(RA_ERR_SHAPE, "n_passes*B*H too large");
+  if ((out_stride_pass % 4) || (out_stride_b % 4) || (out_stride_h % 4) || (out_stride_l % 4))
     return fail(RA_ERR_ALIGN, "out strides must be multiples of 4 elements");
   // the kernel loads 16 bytes of fp32 and stores 8 bytes of bf16 at a time
   if (reinterpret_cast<uintptr_t>(out) % 8u) return fail(RA_ERR_ALIGN, "out must be 8-byte aligned");
   if (!aligned16(acc)) return fail(RA_ERR_ALIGN, "acc is not 16-byte aligned");
-  hipError_t e = ra::launch_bwd_finalize(acc, out, out_stride_b, out_stride_h, out_stride_l, B, H, L,
-                                         D, (hipStream_t)stream);
+  hipError_t e = ra::launch_bwd_finalize(acc, out, out_stride_pass, out_stride_b, out_stride_h, out_stride_l,
+                                         n_passes, B, H, L, D, (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_bwd_finalize launch");
+}
+
+int ra_bwd_finalize(const float* acc, void* out, int64_t out_stride_b, int64_t out_stride_h,
+                    int64_t out_stride_l, int32_t B, int32_t H, int32_t L, int32_t D, void* stream) {
+  return ra_bwd_finalize_passes(acc, out, 0, out_stride_b, out_stride_h, out_stride_l, 1, B, H, L, D, stream);
 }
 
 }  // extern "C"

@@ -21,22 +21,26 @@ constexpr int kBwdMaxListTiles = 2048;
 // ------------------------------------------------------------------------------------------------
 // delta
 // ------------------------------------------------------------------------------------------------
+// n_pass shards per launch: shard p reads out + p * sp and dout.ptr + p * dsp and writes the p-th
+// [B, H, Lq] block of delta.
 template <typename OutT, int D>
-__global__ void bwd_delta_kernel(const OutT* out, long long sb, long long sh, long long sl, TensorArg dout,
-                                 float* delta, int B, int H, int Lq) {
+__global__ void bwd_delta_kernel(const OutT* out, long long sp, long long sb, long long sh, long long sl,
+                                 TensorArg dout, long long dsp, float* delta, int n_pass, int B, int H, int Lq) {
   constexpr int CPR = D / 8;           // lanes per row
   constexpr int RPB = 256 / CPR;       // rows per block
   const int tid = threadIdx.x;
   const long long row = (long long)blockIdx.x * RPB + tid / CPR;
   const int c = tid % CPR;
-  const long long rows = (long long)B * H * Lq;
+  const long long rows = (long long)n_pass * B * H * Lq;
   float acc = 0.f;
   if (row < rows) {
     const int li = (int)(row % Lq);
     const int h = (int)((row / Lq) % H);
-    const int b = (int)(row / ((long long)Lq * H));
-    const OutT* op = out + b * sb + h * sh + (long long)li * sl + 8 * c;
-    const bf16_t* dp = dout.ptr + b * dout.sb + h * dout.sh + (long long)li * dout.sl + 8 * c;
+    const long long bp = row / ((long long)Lq * H);
+    const int b = (int)(bp % B);
+    const long long ps = bp / B;
+    const OutT* op = out + ps * sp + b * sb + h * sh + (long long)li * sl + 8 * c;
+    const bf16_t* dp = dout.ptr + ps * dsp + b * dout.sb + h * dout.sh + (long long)li * dout.sl + 8 * c;
     bf16x8 dv = *(const bf16x8*)dp;
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc += (float)op[e] * (float)dv[e];
@@ -64,11 +68,12 @@ constexpr int kQTile = 32;  // queries per LDS tile in dkdv_kernel
 // (operands visible before the barrier, so their fetch straddles it; the next tile's loads and
 // the hand-over of S(i), dP(i) to the vector ALU issue in their shadow), then the 16 MFMAs of
 // S(i+1) = Q K^T and dP(i+1) = dO V^T with the exp2 / dS arithmetic of tile i in theirs.
-// MULTI: the launch walks the query shards of `shards` one after another (the query side of the
-// ring steps that this key/value shard takes part in); dK / dV stay in registers between them.
+// MULTI: grid dimension y is a ring pass, one key/value shard with its dk / dv.  The launch walks
+// the query shards that `ring` lists for the pass one after another (the query side of the ring
+// steps that this key/value shard takes part in); dK / dV stay in registers between them.
 template <int D, int MODE, bool MULTI>
 __global__ __launch_bounds__(256) void dkdv_kernel(
-    const BwdArgs a, const std::conditional_t<MULTI, QShardList, NoShardList> shards) {
+    const BwdArgs a, const std::conditional_t<MULTI, QRing, NoShardList> ring) {
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int NT = 256;
@@ -103,6 +108,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const BiasArgs& bs = a.bias;
   const int flags = bs.flags;
   const bool wave_on = kw < a.Lk;
+  // the key/value side of this workgroup's pass
+  auto pass_kv_off = [&]() -> int { if constexpr (MULTI) return ring.kv_off[blockIdx.y]; else return bs.kv_off; };
 
   // ---- resident key-side operands ----------------------------------------------------------
   // K is multiplied once, here, by the power of two below sm_scale * log2(e) - exact in bf16 - so
@@ -118,8 +125,18 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   {
     bf16x8 kf[KS], vf[KS];
     const int ki = min(kw + l32, a.Lk - 1);
-    const bf16_t* kp = a.k.ptr + b * a.k.sb + h * a.k.sh + (long long)ki * a.k.sl + 8 * g;
-    const bf16_t* vp = a.v.ptr + b * a.v.sb + h * a.v.sh + (long long)ki * a.v.sl + 8 * g;
+    const bf16_t* k_res = a.k.ptr;
+    const bf16_t* v_res = a.v.ptr;
+    const int* kv_seg_res = bs.kv_seg;
+    const int* kv_pre_res = bs.kv_pre;
+    if constexpr (MULTI) {
+      k_res = ring.k[blockIdx.y];
+      v_res = ring.v[blockIdx.y];
+      kv_seg_res = ring.kv_seg[blockIdx.y];
+      kv_pre_res = ring.kv_pre[blockIdx.y];
+    }
+    const bf16_t* kp = k_res + b * a.k.sb + h * a.k.sh + (long long)ki * a.k.sl + 8 * g;
+    const bf16_t* vp = v_res + b * a.v.sb + h * a.v.sh + (long long)ki * a.v.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       const bf16x8 kr = *(const bf16x8*)(kp + 16 * s);
@@ -127,8 +144,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       for (int e = 0; e < 8; ++e) kf[s][e] = (bf16_t)((float)kr[e] * a.scale_p2);
       vf[s] = *(const bf16x8*)(vp + 16 * s);
     }
-    if (GENERAL && (flags & RA_BIAS_SEGMENT)) k_seg = bs.kv_seg[b * bs.kv_seg_sb + ki];
-    if (GENERAL && (flags & RA_BIAS_PREFIX)) k_pre = bs.kv_pre[b * bs.kv_pre_sb + ki];
+    if (GENERAL && (flags & RA_BIAS_SEGMENT)) k_seg = kv_seg_res[b * bs.kv_seg_sb + ki];
+    if (GENERAL && (flags & RA_BIAS_PREFIX)) k_pre = kv_pre_res[b * bs.kv_pre_sb + ki];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       // an empty statement whose result is bound to accumulation registers: the compiler
@@ -176,17 +193,18 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const int* q_pre_ptr = bs.q_pre;
   const float* dense_ptr = bs.dense;
   int n_shards = 1;
-  if constexpr (MULTI) n_shards = shards.n;
+  if constexpr (MULTI) n_shards = ring.count[blockIdx.y];
   for (int shard = 0; shard < n_shards; ++shard) {
   if constexpr (MULTI) {
-    q_off = shards.q_off[shard];
-    q_ptr = shards.q[shard];
-    do_ptr = shards.dout[shard];
-    lse_ptr = shards.lse[shard];
-    delta_ptr = shards.delta[shard];
-    q_seg_ptr = shards.q_seg[shard];
-    q_pre_ptr = shards.q_pre[shard];
-    dense_ptr = shards.dense[shard];
+    const int si = ring.order[blockIdx.y][shard];
+    q_off = ring.q.q_off[si];
+    q_ptr = ring.q.q[si];
+    do_ptr = ring.q.dout[si];
+    lse_ptr = ring.q.lse[si];
+    delta_ptr = ring.q.delta[si];
+    q_seg_ptr = ring.q.q_seg[si];
+    q_pre_ptr = ring.q.q_pre[si];
+    dense_ptr = ring.q.dense[si];
     // other waves may still be reading the last tile of the previous shard
     if (shard > 0) __syncthreads();
   }
@@ -196,7 +214,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const int ntiles = (a.Lq + kQTile - 1) / kQTile;
   const int k_hi = min(k0 + KEYS_WG, a.Lk) - 1;
   int i_lo, i_hi;
-  query_tile_range(flags, bs.window, bs.kv_off + k0, bs.kv_off + k_hi, q_off, ntiles, kQTile, i_lo, i_hi);
+  const int kv_off = pass_kv_off();
+  query_tile_range(flags, bs.window, kv_off + k0, kv_off + k_hi, q_off, ntiles, kQTile, i_lo, i_hi);
   int n_act = i_hi - i_lo;
   bool use_list = false;
   // ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` that need no segment test
@@ -380,8 +399,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   auto tile_class = [&](int i, int& qt0, int& segbit) -> int {
     qt0 = tile_at(i, segbit) * kQTile;
     if (flags & RA_BIAS_PREFIX) return 2;
-    return classify_pos(flags, bs.window, q_off + qt0, q_off + qt0 + kQTile - 1, bs.kv_off + kw,
-                        bs.kv_off + kw + 31);
+    return classify_pos(flags, bs.window, q_off + qt0, q_off + qt0 + kQTile - 1, kv_off + kw,
+                        kv_off + kw + 31);
   };
   auto needs_bias = [&](int qt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (qt0 + kQTile > a.Lq);
@@ -445,7 +464,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     tb.dense = nullptr;
     tb.dense_vs = 1;
     tb.var_limit = a.Lq - (qt0 + 4 * g);
-    const int rel0 = (q_off + qt0 + 4 * g) - (bs.kv_off + kw + l32);
+    const int rel0 = (q_off + qt0 + 4 * g) - (kv_off + kw + l32);
     const int* ids = (const int*)(stat_rd + ids_buf * STAT_BYTES);
     if (DENSE) {
       tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)(qt0 + 4 * g) * bs.dense_sq +
@@ -472,7 +491,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   int plain_lo = 0, plain_hi = 0;
   if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
-    query_tile_plain_range(flags, bs.window, bs.kv_off + kw, bs.kv_off + kw + 31, q_off, a.Lq / kQTile,
+    query_tile_plain_range(flags, bs.window, kv_off + kw, kv_off + kw + 31, q_off, a.Lq / kQTile,
                            kQTile, lo, hi);
     plain_lo = max(lo - tile_base, run_lo);
     plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
@@ -741,8 +760,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   // All loads of an array are issued before the first value is needed: a load - add - store chain
   // per element would cost one memory round trip each, a hundred in a row with nothing to hide them.
   {
-    float* const dkp = a.dk + (((long long)b * a.H + h) * a.Lk + kw + 4 * g) * D + l32;
-    float* const dvp = a.dv + (((long long)b * a.H + h) * a.Lk + kw + 4 * g) * D + l32;
+    float* dk_res = a.dk;
+    float* dv_res = a.dv;
+    if constexpr (MULTI) {
+      dk_res = ring.dk[blockIdx.y];
+      dv_res = ring.dv[blockIdx.y];
+    }
+    float* const dkp = dk_res + (((long long)b * a.H + h) * a.Lk + kw + 4 * g) * D + l32;
+    float* const dvp = dv_res + (((long long)b * a.H + h) * a.Lk + kw + 4 * g) * D + l32;
     const int key0 = kw + 4 * g;
     auto add_to = [&](float* p, const f32x16 (&acc)[DB], float mul) {
       float old[DB][16];
@@ -787,11 +812,12 @@ constexpr int kDqKeyTile = 32; // keys per LDS tile
 // fetch.  Iteration i, after its barrier, first runs the 8 MFMAs of dQ^T for tile i-1 (operands
 // visible before the barrier, so their fetch straddles it), then the 16 MFMAs of S^T(i+1),
 // dP^T(i+1) with the exp2 / dS arithmetic of tile i in their shadow.
-// MULTI: the launch walks the key/value shards of `shards` one after another (consecutive ring
-// steps of one query shard); dQ stays in registers between them.
+// MULTI: grid dimension y is a ring pass, one query shard with its dq accumulator.  The launch
+// walks the key/value shards that `ring` lists for the pass one after another (consecutive ring
+// steps of that query shard); dQ stays in registers between them.
 template <int D, int MODE, bool MULTI>
 __global__ __launch_bounds__(kDqThreads) void dq_kernel(
-    const BwdArgs a, const std::conditional_t<MULTI, KvShardList, NoShardList> shards) {
+    const BwdArgs a, const std::conditional_t<MULTI, KvRing, NoShardList> ring) {
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;
@@ -834,8 +860,14 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 
   bf16x8 qf[KS], dof[KS];
   {
-    const bf16_t* qp = a.q.ptr + b * a.q.sb + h * a.q.sh + (long long)qi_c * a.q.sl + 8 * g;
-    const bf16_t* dp = a.dout.ptr + b * a.dout.sb + h * a.dout.sh + (long long)qi_c * a.dout.sl + 8 * g;
+    const bf16_t* q_res = a.q.ptr;
+    const bf16_t* do_res = a.dout.ptr;
+    if constexpr (MULTI) {
+      q_res = ring.q[blockIdx.y];
+      do_res = ring.dout[blockIdx.y];
+    }
+    const bf16_t* qp = q_res + b * a.q.sb + h * a.q.sh + (long long)qi_c * a.q.sl + 8 * g;
+    const bf16_t* dp = do_res + b * a.dout.sb + h * a.dout.sh + (long long)qi_c * a.dout.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
       // Q is multiplied once, here, by the power of two below sm_scale * log2(e) (exact in bf16);
@@ -852,9 +884,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     }
   }
   const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
-  const float Lraw = a.lse[row];
+  const float* lse_res = a.lse;
+  const float* delta_res = a.delta;
+  if constexpr (MULTI) {
+    lse_res = ring.x1[blockIdx.y];
+    delta_res = ring.x2[blockIdx.y];
+  }
+  const float Lraw = lse_res[row];
   float neg_lse2 = (Lraw == RA_NEG_INF) ? RA_NEG_INF : -Lraw * kLog2e;  // fully masked row: P = 0
-  float delta = a.delta[row];
+  float delta = delta_res[row];
   // exp2(S - lse2) (dP - delta) = exp2(S) (c dP - c delta) with c = exp2(-lse2): one vector
   // instruction less per score.  Only where no row's logsumexp is so large that exp2(S) or c
   // could leave the fp32 range (S <= lse2 always); other waves have no straight-line stretch.
@@ -869,8 +907,14 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   int q_seg = 0, q_pre = 0;
   float slope2 = 0.f;
   if (GENERAL) {
-    if (flags & RA_BIAS_SEGMENT) q_seg = bs.q_seg[b * bs.q_seg_sb + qi_c];
-    if (flags & RA_BIAS_PREFIX) q_pre = bs.q_pre[b * bs.q_pre_sb + qi_c];
+    const int* q_seg_res = bs.q_seg;
+    const int* q_pre_res = bs.q_pre;
+    if constexpr (MULTI) {
+      q_seg_res = ring.q_seg[blockIdx.y];
+      q_pre_res = ring.q_pre[blockIdx.y];
+    }
+    if (flags & RA_BIAS_SEGMENT) q_seg = q_seg_res[b * bs.q_seg_sb + qi_c];
+    if (flags & RA_BIAS_PREFIX) q_pre = q_pre_res[b * bs.q_pre_sb + qi_c];
     if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e / a.scale_res;
   }
   // ---- one pass of everything below per key/value shard ------------------------------------
@@ -881,15 +925,16 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   const int* kv_pre_ptr = bs.kv_pre;
   const float* dense_ptr = bs.dense;
   int n_shards = 1;
-  if constexpr (MULTI) n_shards = shards.n;
+  if constexpr (MULTI) n_shards = ring.count[blockIdx.y];
   for (int shard = 0; shard < n_shards; ++shard) {
   if constexpr (MULTI) {
-    kv_off = shards.kv_off[shard];
-    k_ptr = shards.k[shard];
-    v_ptr = shards.v[shard];
-    kv_seg_ptr = shards.kv_seg[shard];
-    kv_pre_ptr = shards.kv_pre[shard];
-    dense_ptr = shards.dense[shard];
+    const int si = ring.order[blockIdx.y][shard];
+    kv_off = ring.kv.kv_off[si];
+    k_ptr = ring.kv.k[si];
+    v_ptr = ring.kv.v[si];
+    kv_seg_ptr = ring.kv.kv_seg[si];
+    kv_pre_ptr = ring.kv.kv_pre[si];
+    dense_ptr = ring.kv.dense[si];
     // other waves may still be reading the last K tile of the previous shard
     if (shard > 0) __syncthreads();
   }
@@ -910,7 +955,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   const int ntiles = (a.Lk + kDqKeyTile - 1) / kDqKeyTile;
   const int q_rows_hi = min(q0 + kDqRows, a.Lq) - 1;
   int j_lo, j_hi;
-  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, kv_off, ntiles, kDqKeyTile,
+  int q_off = bs.q_off;
+  if constexpr (MULTI) q_off = ring.q_off[blockIdx.y];
+  key_tile_range(flags, bs.window, q_off + q0, q_off + q_rows_hi, kv_off, ntiles, kDqKeyTile,
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
@@ -1050,7 +1097,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   auto tile_class = [&](int i, int& kt0, int& segbit) -> int {
     kt0 = tile_at(i, segbit) * kDqKeyTile;
     if (flags & RA_BIAS_PREFIX) return 2;
-    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off + kt0,
+    return classify_pos(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off + kt0,
                         kv_off + kt0 + kDqKeyTile - 1);
   };
   auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
@@ -1103,7 +1150,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     tb.dense_vs = 1;
     const int var0 = kt0 + 4 * g;
     tb.var_limit = a.Lk - var0;
-    const int rel0 = (bs.q_off + qi) - (kv_off + var0);
+    const int rel0 = (q_off + qi) - (kv_off + var0);
     if (DENSE)
       tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
     apply_bias<true, DENSE>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
@@ -1137,7 +1184,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   run_tile0 = __builtin_amdgcn_readfirstlane(run_tile0);
   if (wave_on && lse_in_range && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;
-    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
+    key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
     plain_lo = max(lo - run_tile0, run_lo);
     plain_hi = max(min(hi - run_tile0, run_hi), plain_lo);
@@ -1420,7 +1467,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   }
   }  // key/value shards
   if (q_valid) {
-    float* dq = a.dq + row * D + 4 * g;
+    float* dq_res = a.dq;
+    if constexpr (MULTI) dq_res = ring.x0[blockIdx.y];
+    float* dq = dq_res + row * D + 4 * g;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -1437,17 +1486,20 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 // ------------------------------------------------------------------------------------------------
 // fp32 accumulator -> bf16 gradient in the caller's layout
 // ------------------------------------------------------------------------------------------------
-__global__ void bwd_finalize_kernel(const float* acc, bf16_t* out, long long sb, long long sh, long long sl,
-                                    int B, int H, int L, int D) {
+// The accumulators of n_pass shards lie one after another; shard p is written to out + p * sp.
+__global__ void bwd_finalize_kernel(const float* acc, bf16_t* out, long long sp, long long sb, long long sh,
+                                    long long sl, int n_pass, int B, int H, int L, int D) {
   const int cpr = D / 4;
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  const long long rows = (long long)B * H * L;
+  const long long rows = (long long)n_pass * B * H * L;
   if (i >= rows * cpr) return;
   const long long row = i / cpr;
   const int c = (int)(i % cpr);
   const int li = (int)(row % L);
   const int h = (int)((row / L) % H);
-  const int b = (int)(row / ((long long)L * H));
+  const long long bp = row / ((long long)L * H);
+  const int b = (int)(bp % B);
+  out += (bp / B) * sp;
   f32x4 x = *(const f32x4*)(acc + row * D + 4 * c);
   bf16x4 y;
 #pragma unroll
@@ -1458,17 +1510,18 @@ __global__ void bwd_finalize_kernel(const float* acc, bf16_t* out, long long sb,
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long long sh, long long sl,
-                            TensorArg dout, float* delta, int B, int H, int Lq, int D, hipStream_t stream) {
-  const long long rows = (long long)B * H * Lq;
+hipError_t launch_bwd_delta(const void* out, int out_f32, long long sp, long long sb, long long sh, long long sl,
+                            TensorArg dout, long long dsp, float* delta, int n_pass, int B, int H, int Lq, int D,
+                            hipStream_t stream) {
+  const long long rows = (long long)n_pass * B * H * Lq;
   const int rpb = 256 / (D / 8);
   dim3 grid((unsigned)((rows + rpb - 1) / rpb)), block(256);
   if (D == 128) {
-    if (out_f32) hipLaunchKernelGGL((bwd_delta_kernel<float, 128>), grid, block, 0, stream, (const float*)out, sb, sh, sl, dout, delta, B, H, Lq);
-    else hipLaunchKernelGGL((bwd_delta_kernel<bf16_t, 128>), grid, block, 0, stream, (const bf16_t*)out, sb, sh, sl, dout, delta, B, H, Lq);
+    if (out_f32) hipLaunchKernelGGL((bwd_delta_kernel<float, 128>), grid, block, 0, stream, (const float*)out, sp, sb, sh, sl, dout, dsp, delta, n_pass, B, H, Lq);
+    else hipLaunchKernelGGL((bwd_delta_kernel<bf16_t, 128>), grid, block, 0, stream, (const bf16_t*)out, sp, sb, sh, sl, dout, dsp, delta, n_pass, B, H, Lq);
   } else {
-    if (out_f32) hipLaunchKernelGGL((bwd_delta_kernel<float, 64>), grid, block, 0, stream, (const float*)out, sb, sh, sl, dout, delta, B, H, Lq);
-    else hipLaunchKernelGGL((bwd_delta_kernel<bf16_t, 64>), grid, block, 0, stream, (const bf16_t*)out, sb, sh, sl, dout, delta, B, H, Lq);
+    if (out_f32) hipLaunchKernelGGL((bwd_delta_kernel<float, 64>), grid, block, 0, stream, (const float*)out, sp, sb, sh, sl, dout, dsp, delta, n_pass, B, H, Lq);
+    else hipLaunchKernelGGL((bwd_delta_kernel<bf16_t, 64>), grid, block, 0, stream, (const bf16_t*)out, sp, sb, sh, sl, dout, dsp, delta, n_pass, B, H, Lq);
   }
   return hipGetLastError();
 }
@@ -1507,10 +1560,10 @@ hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStre
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QShardList& shards, int D, int mode, hipStream_t stream) {
+hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QRing& shards, int D, int mode, hipStream_t stream) {
   const int keys_wg = 128;
   const int nkt = (a.Lk + keys_wg - 1) / keys_wg;
-  dim3 grid((unsigned)(a.B * a.H * nkt)), block(256);
+  dim3 grid((unsigned)(a.B * a.H * nkt), (unsigned)shards.n_pass), block(256);
   if (D == 128) {
     if (mode == 2) hipLaunchKernelGGL((dkdv_kernel<128, 2, true>), grid, block, 0, stream, a, shards);
     else if (mode == 1) hipLaunchKernelGGL((dkdv_kernel<128, 1, true>), grid, block, 0, stream, a, shards);
@@ -1523,9 +1576,9 @@ hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QShardList& shards, int
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream) {
+hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvRing& shards, int D, int mode, hipStream_t stream) {
   const int nqt = (a.Lq + kDqRows - 1) / kDqRows;
-  dim3 grid((unsigned)(a.B * a.H * nqt)), block(kDqThreads);
+  dim3 grid((unsigned)(a.B * a.H * nqt), (unsigned)shards.n_pass), block(kDqThreads);
   if (D == 128) {
     if (mode == 2) hipLaunchKernelGGL((dq_kernel<128, 2, true>), grid, block, 0, stream, a, shards);
     else if (mode == 1) hipLaunchKernelGGL((dq_kernel<128, 1, true>), grid, block, 0, stream, a, shards);
@@ -1538,11 +1591,11 @@ hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvShardList& shards, int 
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl, int B,
-                               int H, int L, int D, hipStream_t stream) {
-  const long long n = (long long)B * H * L * (D / 4);
+hipError_t launch_bwd_finalize(const float* acc, void* out, long long sp, long long sb, long long sh, long long sl,
+                               int n_pass, int B, int H, int L, int D, hipStream_t stream) {
+  const long long n = (long long)n_pass * B * H * L * (D / 4);
   hipLaunchKernelGGL(bwd_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, acc,
-                     (bf16_t*)out, sb, sh, sl, B, H, L, D);
+                     (bf16_t*)out, sp, sb, sh, sl, n_pass, B, H, L, D);
   return hipGetLastError();
 }
 

@@ -19,12 +19,13 @@ constexpr int kKeyTile = 64;    // keys per LDS tile
 constexpr int kMaxListTiles = 1024;
 constexpr int kPlainMinTiles = 16;  // shortest stretch of plain tiles that takes the straight-line loop
 
-// MULTI: the launch walks the key/value shards of `shards` one after another (the arguments of
-// consecutive ring steps of one query shard); the step's contribution stays in registers
-// between them and meets the carry once, at the end.
+// MULTI: grid dimension y is a ring pass, the trip of one query shard around the ring.  The launch
+// walks the key/value shards that `ring` lists for the pass one after another (the arguments of
+// consecutive ring steps of that query shard); the step's contribution stays in registers between
+// them and meets the carry of the pass once, at the end.
 template <int D, int MODE, bool MULTI>
 __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
-    const FwdArgs a, const std::conditional_t<MULTI, KvShardList, NoShardList> shards) {
+    const FwdArgs a, const std::conditional_t<MULTI, KvRing, NoShardList> ring) {
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;  // k-steps of the QK^T contraction
@@ -59,11 +60,19 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   const int qi_c = min(qi, a.Lq - 1);
   const BiasArgs& bs = a.bias;
   const int flags = bs.flags;
+  // the query side of this workgroup's pass (read from the argument block where it is needed:
+  // nothing of it is carried through the loops)
+  auto pass_q_off = [&]() -> int { if constexpr (MULTI) return ring.q_off[blockIdx.y]; else return bs.q_off; };
+  auto pass_o = [&]() -> float* { if constexpr (MULTI) return ring.x0[blockIdx.y]; else return a.o; };
+  auto pass_m = [&]() -> float* { if constexpr (MULTI) return ring.x1[blockIdx.y]; else return a.m; };
+  auto pass_l = [&]() -> float* { if constexpr (MULTI) return ring.x2[blockIdx.y]; else return a.l; };
 
   // ---- per-lane query state ------------------------------------------------------------
   bf16x8 qf[KS];
   {
-    const bf16_t* qp = a.q.ptr + b * a.q.sb + h * a.q.sh + (long long)qi_c * a.q.sl + 8 * g;
+    const bf16_t* q_ptr = a.q.ptr;
+    if constexpr (MULTI) q_ptr = ring.q[blockIdx.y];
+    const bf16_t* qp = q_ptr + b * a.q.sb + h * a.q.sh + (long long)qi_c * a.q.sl + 8 * g;
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
     if (TIGHT) s_q0[tid] = qf[0];
@@ -76,7 +85,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // l_run / lr_run makes it a properly normalised average of V times the exact row sum, so
   // the rounding of P cancels in o / l instead of showing up as an error of order 2^-9 |v|
   // on rows that see only a few keys.
-  float m_run = a.m[row] * kLog2e;  // exponent reference (log2 domain), moves lazily
+  float m_run = pass_m()[row] * kLog2e;  // exponent reference (log2 domain), moves lazily
   float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
   // In a long stretch of completely unmasked tiles (at least kPlainMinTiles of them) a tile adds
   // only its ROUNDED probabilities, to this third sum, which counts for both l and lr: the
@@ -95,8 +104,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   int q_seg = 0, q_pre = 0;
   float slope2 = 0.f;
   if (GENERAL) {
-    if (flags & RA_BIAS_SEGMENT) q_seg = bs.q_seg[b * bs.q_seg_sb + qi_c];
-    if (flags & RA_BIAS_PREFIX) q_pre = bs.q_pre[b * bs.q_pre_sb + qi_c];
+    const int* q_seg_ptr = bs.q_seg;
+    const int* q_pre_ptr = bs.q_pre;
+    if constexpr (MULTI) {
+      q_seg_ptr = ring.q_seg[blockIdx.y];
+      q_pre_ptr = ring.q_pre[blockIdx.y];
+    }
+    if (flags & RA_BIAS_SEGMENT) q_seg = q_seg_ptr[b * bs.q_seg_sb + qi_c];
+    if (flags & RA_BIAS_PREFIX) q_pre = q_pre_ptr[b * bs.q_pre_sb + qi_c];
     if (flags & RA_BIAS_ALIBI) slope2 = bs.slopes[h] * kLog2e;
   }
   float m_true = m_run;  // exact running maximum; m_run is the (possibly stale) exponent reference
@@ -109,15 +124,16 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   const int* kv_pre_ptr = bs.kv_pre;
   const float* dense_ptr = bs.dense;
   int n_shards = 1;
-  if constexpr (MULTI) n_shards = shards.n;
+  if constexpr (MULTI) n_shards = ring.count[blockIdx.y];
   for (int shard = 0; shard < n_shards; ++shard) {
   if constexpr (MULTI) {
-    kv_off = shards.kv_off[shard];
-    k_ptr = shards.k[shard];
-    v_ptr = shards.v[shard];
-    kv_seg_ptr = shards.kv_seg[shard];
-    kv_pre_ptr = shards.kv_pre[shard];
-    dense_ptr = shards.dense[shard];
+    const int si = ring.order[blockIdx.y][shard];
+    kv_off = ring.kv.kv_off[si];
+    k_ptr = ring.kv.k[si];
+    v_ptr = ring.kv.v[si];
+    kv_seg_ptr = ring.kv.kv_seg[si];
+    kv_pre_ptr = ring.kv.kv_pre[si];
+    dense_ptr = ring.kv.dense[si];
     // the late waves may still be reading the last V tile of the previous shard
     if (shard > 0) __syncthreads();
   }
@@ -136,7 +152,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   const int ntiles = (a.Lk + kKeyTile - 1) / kKeyTile;
   const int q_rows_hi = min(q0 + kFwdRows, a.Lq) - 1;
   int j_lo, j_hi;
-  key_tile_range(flags, bs.window, bs.q_off + q0, bs.q_off + q_rows_hi, kv_off, ntiles, kKeyTile,
+  const int q_off = pass_q_off();
+  key_tile_range(flags, bs.window, q_off + q0, q_off + q_rows_hi, kv_off, ntiles, kKeyTile,
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
@@ -340,7 +357,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   auto tile_class = [&](int i, int& kt0, int& segbit) -> int {
     kt0 = tile_at(i, segbit) * kKeyTile;
     if (flags & RA_BIAS_PREFIX) return 2;
-    return classify_pos(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off + kt0,
+    return classify_pos(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off + kt0,
                         kv_off + kt0 + kKeyTile - 1);
   };
   // Per-lane LDS byte offsets of the operand fetches.  Everything that changes from one MFMA
@@ -439,7 +456,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       for (int r = 0; r < 16; ++r) S[kb][r] *= a.scale2;
       const int var0 = kt0 + 32 * kb + 4 * g;
       tb.var_limit = a.Lk - var0;
-      const int rel0 = (bs.q_off + qi) - (kv_off + var0);
+      const int rel0 = (q_off + qi) - (kv_off + var0);
       if (DENSE)
         tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
       apply_bias<true, DENSE>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
@@ -474,7 +491,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   int plain_lo = 0, plain_hi = 0;
   if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;  // tile indices
-    key_tile_plain_range(flags, bs.window, bs.q_off + qw, bs.q_off + qw + 31, kv_off, a.Lk / kKeyTile,
+    key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kKeyTile,
                          kKeyTile, lo, hi);
     plain_lo = max(lo - tile_base, run_lo);
     plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
@@ -850,17 +867,17 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     // the row index and the incoming maximum are recomputed / reloaded: not worth two registers
     // over the whole loop
     row = ((long long)b * a.H + h) * a.Lq + min(q0 + wave * 32 + l32, a.Lq - 1);
-    const float m_in = a.m[row] * kLog2e;
+    const float m_in = pass_m()[row] * kLog2e;
     const float l_step = half_sum(l_run + lp_run), lr_step = half_sum(lr_run + lp_run);
     const float m_out = m_true;  // started from m_in, so it already covers the carry
     const float m_safe = (m_out == RA_NEG_INF) ? 0.f : m_out;
     const float f_in = fast_exp2(m_in - m_safe);   // 0 for an empty carry
     float f_step = fast_exp2(m_run - m_safe);      // 1 where the reference is exact
     const float ratio = (lr_step > 0.f) ? l_step / lr_step : 1.f;
-    const float l_out = a.l[row] * f_in + l_step * f_step;
+    const float l_out = pass_l()[row] * f_in + l_step * f_step;
     f_step *= ratio;
     if (q_valid) {
-      float* op = a.o + row * D + 4 * g;
+      float* op = pass_o() + row * D + 4 * g;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -871,8 +888,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
           *(f32x4*)(op + 32 * db + 8 * bb) = t;
         }
       if (g == 0) {
-        a.m[row] = m_out * kLn2;
-        a.l[row] = l_out;
+        pass_m()[row] = m_out * kLn2;
+        pass_l()[row] = l_out;
       }
     }
   }
@@ -891,19 +908,23 @@ __global__ void fwd_init_kernel(float* o, float* m, float* l, long long rows, in
   }
 }
 
+// The carries of n_pass query shards lie one after another ([n_pass, B, H, Lq, D]); shard p is
+// written to out + p * sp.
 template <typename OutT>
-__global__ void fwd_finalize_kernel(const float* o, const float* m, const float* l, OutT* out,
-                                    long long sb, long long sh, long long sl, float* lse, int B,
+__global__ void fwd_finalize_kernel(const float* o, const float* m, const float* l, OutT* out, long long sp,
+                                    long long sb, long long sh, long long sl, float* lse, int n_pass, int B,
                                     int H, int Lq, int D) {
   const int cpr = D / 4;
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-  const long long rows = (long long)B * H * Lq;
+  const long long rows = (long long)n_pass * B * H * Lq;
   if (i >= rows * cpr) return;
   const long long row = i / cpr;
   const int c = (int)(i % cpr);
   const int li = (int)(row % Lq);
   const int h = (int)((row / Lq) % H);
-  const int b = (int)(row / ((long long)Lq * H));
+  const long long bp = row / ((long long)Lq * H);
+  const int b = (int)(bp % B);
+  out += (bp / B) * sp;
   const float lv = l[row];
   f32x4 x = *(const f32x4*)(o + row * D + 4 * c);
   typedef __attribute__((ext_vector_type(4))) OutT out4;
@@ -923,9 +944,9 @@ namespace ra {
 
 // mode: 0 = causal / window terms only, 1 = any of the per-tile terms, 2 = a dense bias block too
 template <bool MULTI, typename Shards>
-static hipError_t launch_fwd(const FwdArgs& a, const Shards& sl, int D, int mode, hipStream_t stream) {
+static hipError_t launch_fwd(const FwdArgs& a, const Shards& sl, int n_pass, int D, int mode, hipStream_t stream) {
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
-  dim3 grid((unsigned)(a.B * a.H * nqt)), block(kFwdThreads);
+  dim3 grid((unsigned)(a.B * a.H * nqt), (unsigned)n_pass), block(kFwdThreads);
   if (D == 128) {
     if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<128, 2, MULTI>), grid, block, 0, stream, a, sl);
     else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<128, 1, MULTI>), grid, block, 0, stream, a, sl);
@@ -939,11 +960,11 @@ static hipError_t launch_fwd(const FwdArgs& a, const Shards& sl, int D, int mode
 }
 
 hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream) {
-  return launch_fwd<false>(a, NoShardList{}, D, mode, stream);
+  return launch_fwd<false>(a, NoShardList{}, 1, D, mode, stream);
 }
 
-hipError_t launch_fwd_steps(const FwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream) {
-  return launch_fwd<true>(a, shards, D, mode, stream);
+hipError_t launch_fwd_steps(const FwdArgs& a, const KvRing& ring, int D, int mode, hipStream_t stream) {
+  return launch_fwd<true>(a, ring, ring.n_pass, D, mode, stream);
 }
 
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream) {
@@ -954,16 +975,16 @@ hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, 
 }
 
 hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, void* out, int out_f32,
-                               long long sb, long long sh, long long sl, float* lse, int B, int H,
-                               int Lq, int D, hipStream_t stream) {
-  const long long n = (long long)B * H * Lq * (D / 4);
+                               long long sp, long long sb, long long sh, long long sl, float* lse, int n_pass,
+                               int B, int H, int Lq, int D, hipStream_t stream) {
+  const long long n = (long long)n_pass * B * H * Lq * (D / 4);
   dim3 grid((unsigned)((n + 255) / 256)), block(256);
   if (out_f32)
-    hipLaunchKernelGGL((fwd_finalize_kernel<float>), grid, block, 0, stream, o, m, l, (float*)out, sb,
-                       sh, sl, lse, B, H, Lq, D);
+    hipLaunchKernelGGL((fwd_finalize_kernel<float>), grid, block, 0, stream, o, m, l, (float*)out, sp, sb,
+                       sh, sl, lse, n_pass, B, H, Lq, D);
   else
-    hipLaunchKernelGGL((fwd_finalize_kernel<bf16_t>), grid, block, 0, stream, o, m, l, (bf16_t*)out,
-                       sb, sh, sl, lse, B, H, Lq, D);
+    hipLaunchKernelGGL((fwd_finalize_kernel<bf16_t>), grid, block, 0, stream, o, m, l, (bf16_t*)out, sp,
+                       sb, sh, sl, lse, n_pass, B, H, Lq, D);
   return hipGetLastError();
 }
 

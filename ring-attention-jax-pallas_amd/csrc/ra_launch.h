@@ -56,19 +56,54 @@ struct QShardList {
 };
 struct NoShardList {};
 
+// A launch that covers several ring PASSES at once (grid dimension y = pass): every pass is the
+// trip of one resident shard around the ring, i.e. what one multi-step launch walks.  The
+// travelling shards come from one shared table; a pass lists the entries it meets, in ring order
+// (steps that are masked entirely are left out by the host).  The resident side of a pass - for
+// the forward and dQ kernels a query shard with its carry or dq accumulator, for the dK/dV kernel
+// a key/value shard with its dk / dv - replaces the corresponding fields of FwdArgs / BwdArgs.
+constexpr int kMaxPasses = 16;
+struct KvRing {
+  KvShardList kv;  // the key/value shards the passes draw from
+  int n_pass;
+  unsigned char count[kMaxPasses];              // live steps of pass p
+  unsigned char order[kMaxPasses][kMaxShards];  // their entries of `kv`, in ring order
+  int q_off[kMaxPasses];
+  const bf16_t* q[kMaxPasses];
+  const bf16_t* dout[kMaxPasses];  // dQ only
+  float* x0[kMaxPasses];           // forward: o carry;  dQ: dq accumulator
+  float* x1[kMaxPasses];           // forward: m;        dQ: lse
+  float* x2[kMaxPasses];           // forward: l;        dQ: delta
+  const int* q_seg[kMaxPasses];
+  const int* q_pre[kMaxPasses];
+};
+struct QRing {
+  QShardList q;  // the query shards the passes draw from
+  int n_pass;
+  unsigned char count[kMaxPasses];
+  unsigned char order[kMaxPasses][kMaxShards];
+  int kv_off[kMaxPasses];
+  const bf16_t* k[kMaxPasses];
+  const bf16_t* v[kMaxPasses];
+  float* dk[kMaxPasses];
+  float* dv[kMaxPasses];
+  const int* kv_seg[kMaxPasses];
+  const int* kv_pre[kMaxPasses];
+};
+
 hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream);
-hipError_t launch_fwd_steps(const FwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream);
+hipError_t launch_fwd_steps(const FwdArgs& a, const KvRing& ring, int D, int mode, hipStream_t stream);
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream);
 hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, void* out, int out_f32,
-                               long long sb, long long sh, long long sl, float* lse, int B, int H,
-                               int Lq, int D, hipStream_t stream);
-hipError_t launch_bwd_delta(const void* out, int out_f32, long long sb, long long sh, long long sl,
-                            TensorArg dout, float* delta, int B, int H, int Lq, int D,
+                               long long sp, long long sb, long long sh, long long sl, float* lse, int n_pass,
+                               int B, int H, int Lq, int D, hipStream_t stream);
+hipError_t launch_bwd_delta(const void* out, int out_f32, long long sp, long long sb, long long sh, long long sl,
+                            TensorArg dout, long long dsp, float* delta, int n_pass, int B, int H, int Lq, int D,
                             hipStream_t stream);
 hipError_t launch_bwd_step(const BwdArgs& a, int D, int mode, int parts, hipStream_t stream);
-hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvShardList& shards, int D, int mode, hipStream_t stream);
-hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QShardList& shards, int D, int mode, hipStream_t stream);
-hipError_t launch_bwd_finalize(const float* acc, void* out, long long sb, long long sh, long long sl,
-                               int B, int H, int L, int D, hipStream_t stream);
+hipError_t launch_bwd_dq_steps(const BwdArgs& a, const KvRing& ring, int D, int mode, hipStream_t stream);
+hipError_t launch_bwd_dkdv_steps(const BwdArgs& a, const QRing& ring, int D, int mode, hipStream_t stream);
+hipError_t launch_bwd_finalize(const float* acc, void* out, long long sp, long long sb, long long sh, long long sl,
+                               int n_pass, int B, int H, int L, int D, hipStream_t stream);
 
 }  // namespace ra

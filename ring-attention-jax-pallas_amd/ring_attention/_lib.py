@@ -74,6 +74,17 @@ EXPORTS = {
     "ra_bwd_step_parts": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
     "ra_bwd_dq_steps": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
     "ra_bwd_dkdv_steps": (C.c_int, [C.POINTER(RaBwdStepParams), C.c_int32, C.c_void_p]),
+    "ra_fwd_passes": (C.c_int, [C.POINTER(RaFwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p]),
+    "ra_bwd_dq_passes": (C.c_int, [C.POINTER(RaBwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p]),
+    "ra_bwd_dkdv_passes": (C.c_int, [C.POINTER(RaBwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p]),
+    "ra_fwd_finalize_passes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64,
+                                         C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int32,
+                                         C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "ra_bwd_delta_passes": (C.c_int, [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                      C.POINTER(RaTensor), C.c_int64, C.c_void_p, C.c_int32, C.c_int32, C.c_int32,
+                                      C.c_int32, C.c_int32, C.c_void_p]),
+    "ra_bwd_finalize_passes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                                         C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "ra_bwd_finalize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32,
                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "ra_step_is_skippable": (C.c_int, [C.POINTER(RaBias), C.c_int32, C.c_int32]),

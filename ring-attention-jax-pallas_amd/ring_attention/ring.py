@@ -36,8 +36,9 @@ from . import _lib
 from .bias import BiasFn, BlockBias
 
 # "hip": one launch per ring step, the reference's loop; "pallas" is accepted as an alias (the
-# fused-kernel choice there).  "hip_fused": one launch per ring PASS - the kernels walk the shards
-# of a query (or key/value) shard's whole trip around the ring themselves.
+# fused-kernel choice there).  "hip_fused": one launch for ALL ring passes - the kernels walk the
+# shards of a query (or key/value) shard's whole trip around the ring themselves, one grid row per
+# resident shard.
 _IMPLS = ("hip", "pallas", "hip_fused")
 
 
@@ -468,118 +469,121 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
     return out, lse
 
 
-_MAX_LANES = 2
-_lane_streams = {}
-
-
-def _lane_count(plan: "_RingPlan", device) -> int:
-    """Two lanes while one pass leaves compute units idle (its forward / dQ grid, one workgroup of
-    256 query rows per compute unit at a time, is smaller than two rounds of the chip); passes
-    that fill the GPU on their own run faster one after the other (measured: 8 shards of 1024
-    tokens gain a third from the second stream, 8 shards of 16384 lose 2 %)."""
-    cus = torch.cuda.get_device_properties(device).multi_processor_count
-    workgroups = plan.B * plan.H * ((plan.Lq + 255) // 256)
-    return _MAX_LANES if workgroups < 2 * cus else 1
-
-
-def _run_in_lanes(jobs, costs, n_lanes):
-    """The ring passes of different shards do not depend on each other: spread them over
-    ``n_lanes`` side streams (longest first, each to the lane with the least work so far) so that
-    launches too small to fill the GPU overlap.  ``jobs[j](lane)`` issues pass j on the current
-    stream using lane-private scratch ``lane``.  The caller's stream waits for all of them."""
-    if n_lanes == 1:
-        for job in jobs:
-            job(0)
-        return
-    main = torch.cuda.current_stream()
-    dev = main.device
-    if dev not in _lane_streams:
-        _lane_streams[dev] = [torch.cuda.Stream(device=dev) for _ in range(_MAX_LANES)]
-    lanes = _lane_streams[dev][:n_lanes]
-    for st in lanes:
-        st.wait_stream(main)
-    load = [0.0] * n_lanes
-    for j in sorted(range(len(jobs)), key=lambda j: -costs[j]):
-        i = load.index(min(load))
-        load[i] += costs[j]
-        with torch.cuda.stream(lanes[i]):
-            jobs[j](i)
-    for st in lanes:
-        main.wait_stream(st)
+def _pass_steps(plan: "_RingPlan", cache_key, key, build):
+    """The parameter blocks of all ring passes of one kind, built once per plan and set of input
+    tensors: only the pointers of buffers allocated per call are patched afterwards."""
+    cache = plan.__dict__.setdefault("_step_cache", {})
+    hit = cache.get(cache_key)
+    if hit is None or hit[0] != key:
+        hit = (key,) + build()
+        cache[cache_key] = hit
+    return hit[1:]
 
 
 def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO_TIMER):
-    """``_ring_forward`` with the whole ring pass of a query shard in one launch: the kernel
-    visits the key/value shards in ring order itself.  Passes too small to fill the GPU run
-    on two streams (``_lane_count``)."""
+    """``_ring_forward`` with ALL ring passes in one launch: grid dimension y is the query shard,
+    and the kernel visits that shard's key/value shards in ring order itself.  Three launches per
+    forward: carry reset, the ring, finalisation."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
+    lib = _lib.load()
     out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
     lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    n_lanes = _lane_count(plan, dev)
-    carry = [init_carry(B, H, Lq, D, dev) for _ in range(n_lanes)]
-    fresh = [True] * n_lanes
+    o = torch.empty((n, B, H, Lq, D), dtype=torch.float32, device=dev)
+    m = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    l = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    _lib.check("ra_fwd_init", lib.ra_fwd_init(o.data_ptr(), m.data_ptr(), l.data_ptr(), n * B, H, Lq, D, _stream()))
 
-    def job(r):
-        def run(lane):
-            o, m, l = carry[lane]
-            if not fresh[lane]:
-                reset_carry(o, m, l)
-            fresh[lane] = False
-            order = [(r - t) % n for t in range(n)]  # ring.py:51-55
-            with timer.span("fwd_pass", r, -1):
-                fwd_blocks(_shard_bhld(q, r, Lq), [(_shard_bhld(k, s, Lk), _shard_bhld(v, s, Lk)) for s in order],
-                           [plan.block_bias(r, s) for s in order], o, m, l, sm_scale)
-            finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
-        return run
+    def build():
+        steps = (_lib.RaFwdStepParams * (n * n))()
+        keep = []  # the bias structs point into tensors that must outlive the calls
+        for r in range(n):
+            for t in range(n):
+                src = (r - t) % n  # ring.py:51-55
+                bias = plan.block_bias(r, src)
+                keep.append(bias)
+                steps[r * n + t] = _fwd_params(_shard_bhld(q, r, Lq), _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk),
+                                               bias, o[r], m[r], l[r], sm_scale)
+        return steps, (C.c_int32 * n)(*([n] * n)), keep
 
-    _run_in_lanes([job(r) for r in range(n)], [plan.live_steps(r, None) for r in range(n)], n_lanes)
+    key = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(), k.stride(), v.stride(), sm_scale)
+    steps, counts, _keep = _pass_steps(plan, "fwd", key, build)
+    if plan.callable is not None:
+        steps, counts, _keep = build()  # a callable's dense blocks are fresh tensors every time
+    so, sm = o[0].numel() * 4, m[0].numel() * 4
+    for r in range(n):
+        for t in range(n):
+            st = steps[r * n + t]
+            st.o, st.m, st.l = o.data_ptr() + r * so, m.data_ptr() + r * sm, l.data_ptr() + r * sm
+    with timer.span("fwd_ring", -1, -1):
+        _lib.check("ra_fwd_passes", lib.ra_fwd_passes(steps, counts, n, _stream()))
+    dt = {torch.bfloat16: _lib.RA_DTYPE_BF16, torch.float32: _lib.RA_DTYPE_F32}[out.dtype]
+    ov = out.permute(0, 2, 1, 3)  # [b, h, S, d] view; shard r starts r * Lq rows further
+    _lib.check("ra_fwd_finalize_passes", lib.ra_fwd_finalize_passes(
+        o.data_ptr(), m.data_ptr(), l.data_ptr(), out.data_ptr(), dt, Lq * ov.stride(2), ov.stride(0), ov.stride(1),
+        ov.stride(2), lse.data_ptr(), n, B, H, Lq, D, _stream()))
     return out, lse
 
 
 def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
-    """``_ring_backward`` with one launch per key/value shard for dK / dV (the kernel visits the
-    query shards in the order they arrive, ring.py:195) and one per query shard for dQ; the
-    launches are independent of each other and, when small, run on two streams."""
+    """``_ring_backward`` with all passes of a kind in one launch: one for dK / dV (grid dimension y
+    is the key/value shard, the kernel visits the query shards in the order they arrive,
+    ring.py:195), one for dQ (y is the query shard), around one delta launch and three casts."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
+    lib = _lib.load()
     delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    for s in range(n):
-        precompute_delta(_shard_bhld(out, s, Lq), _shard_bhld(do, s, Lq), delta[s])
+    ov, dov = out.permute(0, 2, 1, 3), do.permute(0, 2, 1, 3)
+    dt = {torch.bfloat16: _lib.RA_DTYPE_BF16, torch.float32: _lib.RA_DTYPE_F32}[out.dtype]
+    do_t = _view_bhld(dov)
+    _lib.check("ra_bwd_delta_passes", lib.ra_bwd_delta_passes(
+        out.data_ptr(), dt, Lq * ov.stride(2), ov.stride(0), ov.stride(1), ov.stride(2), C.byref(do_t),
+        Lq * dov.stride(2), delta.data_ptr(), n, B, H, Lq, D, _stream()))
     dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
-    n_lanes = _lane_count(plan, dev)
-    dkv_acc = [(torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev),
-                torch.empty((B, H, Lk, D), dtype=torch.float32, device=dev)) for _ in range(n_lanes)]
+    dkv_acc = torch.zeros((2, n, B, H, Lk, D), dtype=torch.float32, device=dev)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
-    def step(qs, ks, dk_acc, dv_acc):
-        return (_shard_bhld(q, qs, Lq), _shard_bhld(k, ks, Lk), _shard_bhld(v, ks, Lk),
-                _shard_bhld(do, qs, Lq), lse[qs], delta[qs], dq_acc[qs], dk_acc, dv_acc,
-                plan.block_bias(qs, ks))
+    def build():
+        by_kv = (_lib.RaBwdStepParams * (n * n))()
+        by_q = (_lib.RaBwdStepParams * (n * n))()
+        keep = []
+        for r in range(n):
+            for t in range(n):
+                # dK / dV: key/value shard r meets query shard (r - t) mod n at step t (ring.py:195);
+                # dQ: query shard r meets key/value shard (r + t) mod n at step t of that device
+                for arr, qs, ks in ((by_kv, (r - t) % n, r), (by_q, r, (r + t) % n)):
+                    bias = plan.block_bias(qs, ks)
+                    keep.append(bias)
+                    arr[r * n + t] = _bwd_params(_shard_bhld(q, qs, Lq), _shard_bhld(k, ks, Lk), _shard_bhld(v, ks, Lk),
+                                                 _shard_bhld(do, qs, Lq), lse[qs], delta[qs], dq_acc[qs],
+                                                 dkv_acc[0, ks], dkv_acc[1, ks], bias, sm_scale)
+        pairs = [((r - t) % n, r) for r in range(n) for t in range(n)], [(r, (r + t) % n) for r in range(n) for t in range(n)]
+        return by_kv, by_q, pairs, (C.c_int32 * n)(*([n] * n)), keep
 
-    def dkdv_job(r):
-        def run(lane):
-            dk_acc, dv_acc = dkv_acc[lane]
-            dk_acc.zero_()
-            dv_acc.zero_()
-            with timer.span("bwd_dkdv_pass", -1, r):
-                _bwd_steps("dkdv", [step((r - t) % n, r, dk_acc, dv_acc) for t in range(n)], sm_scale)
-            _finalize_grad(dk_acc, _shard_bhld(dk, r, Lk))
-            _finalize_grad(dv_acc, _shard_bhld(dv, r, Lk))
-        return run
-
-    def dq_job(s):
-        def run(lane):
-            dk_acc, dv_acc = dkv_acc[lane]  # not touched by a dQ launch
-            # query shard s meets key/value shard r at step (r - s) mod n of device r
-            with timer.span("bwd_dq_pass", s, -1):
-                _bwd_steps("dq", [step(s, (s + t) % n, dk_acc, dv_acc) for t in range(n)], sm_scale)
-            _finalize_grad(dq_acc[s], _shard_bhld(dq, s, Lq))
-        return run
-
-    jobs = [dkdv_job(r) for r in range(n)] + [dq_job(s) for s in range(n)]
-    costs = [8.0 * plan.live_steps(None, r) for r in range(n)] + [6.0 * plan.live_steps(s, None) for s in range(n)]
-    _run_in_lanes(jobs, costs, n_lanes)
+    key = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(), k.stride(), v.stride(), do.stride(), sm_scale)
+    by_kv, by_q, pairs, counts, _keep = _pass_steps(plan, "bwd", key, build)
+    if plan.callable is not None:
+        by_kv, by_q, pairs, counts, _keep = build()
+    s_row, s_acc, s_kv = lse[0].numel() * 4, dq_acc[0].numel() * 4, dkv_acc[0, 0].numel() * 4
+    do_shard = Lq * do.stride(1) * do.element_size()
+    for arr, pr in zip((by_kv, by_q), pairs):
+        for i, (qs, ks) in enumerate(pr):
+            st = arr[i]
+            st.dout.ptr = do.data_ptr() + qs * do_shard
+            st.dout.stride_b, st.dout.stride_h, st.dout.stride_l = do.stride(0), do.stride(2), do.stride(1)
+            st.lse, st.delta = lse.data_ptr() + qs * s_row, delta.data_ptr() + qs * s_row
+            st.dq = dq_acc.data_ptr() + qs * s_acc
+            st.dk = dkv_acc.data_ptr() + ks * s_kv
+            st.dv = dkv_acc.data_ptr() + (n + ks) * s_kv
+    with timer.span("bwd_dkdv_ring", -1, -1):
+        _lib.check("ra_bwd_dkdv_passes", lib.ra_bwd_dkdv_passes(by_kv, counts, n, _stream()))
+    with timer.span("bwd_dq_ring", -1, -1):
+        _lib.check("ra_bwd_dq_passes", lib.ra_bwd_dq_passes(by_q, counts, n, _stream()))
+    for acc, g, L in ((dq_acc, dq, Lq), (dkv_acc[0], dk, Lk), (dkv_acc[1], dv, Lk)):
+        gv = g.permute(0, 2, 1, 3)
+        _lib.check("ra_bwd_finalize_passes", lib.ra_bwd_finalize_passes(
+            acc.data_ptr(), g.data_ptr(), L * gv.stride(2), gv.stride(0), gv.stride(1), gv.stride(2), n, B, H, L, D,
+            _stream()))
     return dq, dk, dv
 
 
@@ -692,7 +696,7 @@ def ring_attention(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = 
             ``kv_`` twins.
         sm_scale: softmax scale, 1/sqrt(d) if unspecified.
         block_impl: ``"hip"`` (one kernel launch per ring step; ``"pallas"`` is accepted as an
-            alias) or ``"hip_fused"`` (one launch per ring pass: the kernels walk the shards
+            alias) or ``"hip_fused"`` (one launch for all ring passes: the kernels walk the shards
             themselves, which pays when shards are small); anything else raises ``ValueError`` as
             the reference does (ring.py:312).
     Returns:

@@ -508,16 +508,51 @@ def _fused_cases():
 
 @pytest.mark.parametrize("name", sorted(_fused_cases()))
 def test_fused_ring_pass(device, name):
-    """block_impl="hip_fused": one launch per ring pass, the kernels walk the shards themselves.
-    Same oracle, same tolerances as the launch-per-step path."""
+    """block_impl="hip_fused": all ring passes in one launch, the kernels walk the shards
+    themselves.  Same oracle, same tolerances as the launch-per-step path."""
     _check(device, "fused " + name, impl="hip_fused", **_fused_cases()[name])
 
 
-def test_fused_ring_pass_on_one_stream(device, monkeypatch):
-    # passes that fill the GPU on their own are issued one after the other on the caller's stream
-    monkeypatch.setattr(rr, "_MAX_LANES", 1)
-    _check(device, "fused, one stream", impl="hip_fused", **_fused_cases()["causal_d128_ring8"])
-    _check(device, "fused, one stream", impl="hip_fused", **_fused_cases()["segments_sorted"])
+def test_pass_entry_points_equal_launches_per_pass(device):
+    """ra_fwd_passes / ra_bwd_dq_passes / ra_bwd_dkdv_passes (all ring passes in one grid) give what
+    one ra_*_steps launch per pass gives, bit for bit: the same workgroups do the same arithmetic."""
+    B, H, D, n, L = 2, 2, 128, 4, 384
+    S = n * L
+    q, k, v, do = (_dev(x, device, torch.bfloat16) for x in R.make_inputs(19, B, S, S, H, D))
+    seg = _dev(R.geometric_segment_ids(2, B, S, 300), device)
+    plan = rr._RingPlan(q, k, n, ra.causal_bias() + ra.segment_bias(), {"q_segment_ids": seg}, {"kv_segment_ids": seg})
+    sc = 1 / math.sqrt(D)
+    sh = lambda x, s_: rr._shard_bhld(x, s_, L)
+    out, lse = rr._ring_forward_fused(q, k, v, plan, sc, torch.float32)
+    dq, dk, dv = rr._ring_backward_fused(q, k, v, out, lse, do, plan, sc)
+    # the same passes, one launch each
+    out1 = torch.empty_like(out)
+    lse1 = torch.empty_like(lse)
+    for r in range(n):
+        o, m, l = rr.init_carry(B, H, L, D, device)
+        order = [(r - t) % n for t in range(n)]
+        rr.fwd_blocks(sh(q, r), [(sh(k, s_), sh(v, s_)) for s_ in order], [plan.block_bias(r, s_) for s_ in order], o, m, l, sc)
+        rr.finalize_carry(o, m, l, sh(out1, r), lse1[r])
+    assert torch.equal(out, out1) and torch.equal(lse, lse1)
+    delta = torch.stack([rr.precompute_delta(sh(out, s_), sh(do, s_)) for s_ in range(n)])
+    z = lambda: torch.zeros((B, H, L, D), dtype=torch.float32, device=device)
+    dq1, dk1, dv1 = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    for r in range(n):
+        dqa, dka, dva = z(), z(), z()
+        rr._bwd_steps("dkdv", [(sh(q, (r - t) % n), sh(k, r), sh(v, r), sh(do, (r - t) % n), lse[(r - t) % n],
+                                delta[(r - t) % n], dqa, dka, dva, plan.block_bias((r - t) % n, r)) for t in range(n)], sc)
+        rr._finalize_grad(dka, sh(dk1, r))
+        rr._finalize_grad(dva, sh(dv1, r))
+        dqa = z()
+        rr._bwd_steps("dq", [(sh(q, r), sh(k, (r + t) % n), sh(v, (r + t) % n), sh(do, r), lse[r], delta[r], dqa, dka, dva,
+                              plan.block_bias(r, (r + t) % n)) for t in range(n)], sc)
+        rr._finalize_grad(dqa, sh(dq1, r))
+    torch.cuda.synchronize()
+    assert torch.equal(dq, dq1) and torch.equal(dk, dk1) and torch.equal(dv, dv1)
+    # a second call reuses the cached parameter blocks of the plan with fresh buffers
+    out2, lse2 = rr._ring_forward_fused(q, k, v, plan, sc, torch.float32)
+    g2 = rr._ring_backward_fused(q, k, v, out2, lse2, do, plan, sc)
+    assert torch.equal(out2, out) and all(torch.equal(a, b_) for a, b_ in zip(g2, (dq, dk, dv)))
 
 
 def test_fused_ring_pass_with_a_callable_bias_fn(device):
