@@ -44,6 +44,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // first operand fragment of Q waits here and is fetched once per iteration instead.
   constexpr bool TIGHT = GENERAL || MULTI;
   __shared__ __attribute__((aligned(16))) bf16x8 s_q0[TIGHT ? kFwdThreads : 1];
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q1[GENERAL ? kFwdThreads : 1];  // the second one too
+  // ALiBi inside the straight-line loop (see plain_iteration): the key-side operand of the extra
+  // matrix instruction, one fragment per 32-key block and lane
+  __shared__ __attribute__((aligned(16))) bf16x8 s_ramp[GENERAL ? 2 : 1][GENERAL ? 64 : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -76,6 +80,22 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
     if (TIGHT) s_q0[tid] = qf[0];
+    if (GENERAL) s_q1[tid] = qf[1];
+    if (GENERAL && tid < 64) {
+      // row (32 kb + l32) of the 32 x 16 operand is [j, j, 1, 1, 0 ...] with j the key's index in
+      // the tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        bf16x8 rf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rf[e] = (bf16_t)0.f;
+        if (g == 0) {
+          rf[0] = rf[1] = (bf16_t)(float)(32 * kb + l32);
+          rf[2] = rf[3] = (bf16_t)1.0f;
+        }
+        s_ramp[kb][tid] = rf;
+      }
+    }
   }
   long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
   // This step accumulates its own contribution from zero and is merged with the incoming carry
@@ -157,11 +177,16 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
-  // ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` that need no segment test
+  // Ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` whose 64 keys share one
+  // segment id each (not necessarily the same one, nor that of every query of the workgroup): the
+  // straight-line loop walks them with one comparison per lane and tile - the lane's query row
+  // belongs to the tile's document or it does not.  wg_one_doc: all queries of the workgroup
+  // share one id, so that a listed tile with one id needs no test at all.
   int run_lo = 0, run_hi = n_act, tile_base = j_lo;
+  bool wg_one_doc = true;
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     // segment-id range of the workgroup's queries, then one thread per key tile decides
-    // whether the id ranges can intersect (skip otherwise) and whether the tile is uniform
+    // whether the id ranges can intersect (skip otherwise) and whether the tile has one id
     use_list = true;
     int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
     smin = wave_min(smin);
@@ -181,9 +206,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       int kmin, kmax;
       tile_id_range<kKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
       const bool act = !(kmax < qmin || kmin > qmax);
-      const bool uniform = (kmin == kmax) && (qmin == qmax) && (kmin == qmin);
-      s_flag[j - j_lo] = act ? (uniform ? 1 : 3) : 0;
+      s_flag[j - j_lo] = act ? ((kmin == kmax) ? 1 : 3) : 0;
     }
+    wg_one_doc = qmin == qmax;
     __syncthreads();
     if (wave == 0) {
       int cnt = 0;
@@ -217,7 +242,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
       int e = s_list[i];
-      segbit = e >> 15;
+      segbit = (e >> 15) | (wg_one_doc ? 0 : 1);  // a tile of several ids, or queries of several
       return e & 0x7fff;
     }
     segbit = 0;
@@ -436,7 +461,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
     return nb;
   };
-  // scale + bias with the id arrays of LDS slot `ids_buf`; returns the row maximum
+  // Bias of a fresh tile with the id arrays of LDS slot `ids_buf`; returns the row maximum (log2
+  // units).  The tile keeps the units of the matrix product: a bias value enters divided by
+  // scale2, so that biased and unbiased tiles go through the same exp2(S * scale2 - m) chain.
   auto prepare = [&](f32x16 (&S)[2], int kt0, int segbit, int cls, int ids_buf) -> float {
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
@@ -445,15 +472,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       if (segbit) tb.flags |= RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
-    tb.slope2 = slope2;
-    tb.dense_mul = kLog2e;
+    const float inv_scale2 = 1.0f / a.scale2;
+    tb.slope2 = slope2 * inv_scale2;
+    tb.dense_mul = kLog2e * inv_scale2;
     tb.dense = nullptr;
     tb.dense_vs = 1;
     float mx = RA_NEG_INF;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) S[kb][r] *= a.scale2;
       const int var0 = kt0 + 32 * kb + 4 * g;
       tb.var_limit = a.Lk - var0;
       const int rel0 = (q_off + qi) - (kv_off + var0);
@@ -464,7 +490,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
     }
-    return half_max(mx);
+    return half_max(mx) * a.scale2;
   };
   // move the exponent reference if some row's maximum outgrew it by more than 2^8; until then
   // probabilities are taken relative to the old reference (they stay below 256, harmless in
@@ -486,18 +512,34 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
   };
 
-  // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
-  // range: they take the fused path without any per-tile classification.
-  int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
+  // Ordinals [st_lo[s], st_hi[s]) of the tiles this wave sees completely, unmasked and in range:
+  // they take the straight-line path without any per-tile classification.  Under ALiBi a stretch
+  // must also lie on one side of the diagonal, where -slope |q_pos - kv_pos| is linear in both
+  // positions (stretch 0: keys before the wave's queries, stretch 1: keys after them).
+  constexpr int NST = 2;
+  const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
+  int st_lo[2] = {0, 0}, st_hi[2] = {0, 0};
+  if (wave_on && !(GENERAL && (flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;  // tile indices
     key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kKeyTile,
                          kKeyTile, lo, hi);
-    plain_lo = max(lo - tile_base, run_lo);
-    plain_hi = max(min(hi - tile_base, run_hi), plain_lo);
+    int lo2 = hi, hi1 = hi;
+    if (alibi_on) {
+      // the same bounds for all waves (the workgroup's first and last query): the waves meet at a
+      // barrier per tile, so a generic iteration in one of them holds up all
+      hi1 = min(hi, floor_div(q_off + q0 - kv_off - (kKeyTile - 1), kKeyTile) + 1);       // last key <= first query
+      lo2 = max(lo, ceil_div(q_off + q0 + kFwdRows - 1 - kv_off, kKeyTile));              // first key >= last query
+    }
+    st_lo[0] = max(lo - tile_base, run_lo);
+    st_hi[0] = max(min(hi1 - tile_base, run_hi), st_lo[0]);
+    st_lo[1] = max(max(lo2 - tile_base, run_lo), st_hi[0]);
+    st_hi[1] = max(min(hi - tile_base, run_hi), st_lo[1]);
   }
-  plain_lo = __builtin_amdgcn_readfirstlane(plain_lo);  // wave-uniform; now the compiler knows
-  plain_hi = __builtin_amdgcn_readfirstlane(plain_hi);
+#pragma unroll
+  for (int st = 0; st < 2; ++st) {  // wave-uniform; now the compiler knows
+    st_lo[st] = __builtin_amdgcn_readfirstlane(st_lo[st]);
+    st_hi[st] = __builtin_amdgcn_readfirstlane(st_hi[st]);
+  }
 
   // Barrier number k and the requests that follow it (see the loop description above).
   const bool late_half = wave_u >= 4;
@@ -516,7 +558,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 
   // per-tile state handed from one iteration to the next
   f32x16 sa[2], sb[2];
-  bool cur_valid = false, cur_scaled = false;
+  bool cur_valid = false;
   float cur_mx = RA_NEG_INF;
   if (n > 0 && wave_on) {
     int kt0, segbit;
@@ -524,8 +566,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (!(cls & 1)) {
       cur_valid = true;
       compute_s(sa, s_k[0]);
-      cur_scaled = needs_bias(kt0, segbit, cls);
-      cur_mx = cur_scaled ? prepare(sa, kt0, segbit, cls, 0) : raw_rowmax(sa);
+      cur_mx = needs_bias(kt0, segbit, cls) ? prepare(sa, kt0, segbit, cls, 0) : raw_rowmax(sa);
     }
   }
 
@@ -536,17 +577,17 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const char* kt = s_k[(PAR + 1) & 3];
     const unsigned vt = PAR * TILE_BYTES;
     int nkt0 = 0, nsegbit = 0, ncls = 1;
-    bool nxt_valid = false, nxt_scaled = false;
-    if (i + 1 >= plain_lo && i + 1 < plain_hi) {
-      nxt_valid = true;
+    bool nxt_valid = false, nxt_biased = false;
+    if (!alibi_on && wg_one_doc && i + 1 >= st_lo[0] && i + 1 < st_hi[0]) {
+      nxt_valid = true;  // inside a stretch of plain tiles (without ALiBi there is one stretch)
     } else if (i + 1 < n && wave_on) {
       ncls = tile_class(i + 1, nkt0, nsegbit);
       nxt_valid = !(ncls & 1);
-      nxt_scaled = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
+      nxt_biased = nxt_valid && needs_bias(nkt0, nsegbit, ncls);
     }
     float nxt_mx = RA_NEG_INF;
     bf16x8 pfrag[4];
-    const bool fused = cur_valid && nxt_valid && !cur_scaled;
+    const bool fused = cur_valid && nxt_valid;
     if (cur_valid) update_reference(cur_mx);
     const float neg_m = (m_run == RA_NEG_INF) ? 0.f : -m_run;
     if (fused) {
@@ -630,7 +671,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float p = cur_scaled ? fast_exp2(SC[kb][r] + neg_m) : fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
+            const float p = fast_exp2(fmaf(SC[kb][r], a.scale2, neg_m));
             SC[kb][r] = p;
             rs += p;
           }
@@ -653,12 +694,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       request_v(i + v_ahead, 0);
       request_v(i + v_ahead, 1);
       if (cur_valid) compute_pv(pfrag, vt);
-      if (nxt_valid && !nxt_scaled) nxt_mx = raw_rowmax(SN);
+      if (nxt_valid && !nxt_biased) nxt_mx = raw_rowmax(SN);
     }
-    if (nxt_scaled) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, (i + 1) & 3);
+    if (nxt_biased) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, (i + 1) & 3);
     if (i + 3 < n) store_ids((i + 3) & 3);
     cur_valid = nxt_valid;
-    cur_scaled = nxt_scaled;
     cur_mx = nxt_mx;
   };
 
@@ -679,6 +719,15 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));  // only the previous barrier's requests are in flight
     __syncthreads();
   };
+  const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
+  // The key-side ids seen through the constant address space: with a wave-uniform index the
+  // compiler fetches them through the scalar cache and tracks the load in flight itself (the
+  // array is not written while the kernel runs).
+  typedef const __attribute__((address_space(4))) int* const_ids;
+  const const_ids doc_ids = (const_ids)(uintptr_t)kv_seg;
+  int doc_cur = 0, doc_nxt = 0, doc_far = 0;  // segment ids of tiles i, i + 1, i + 2 of a stretch
+  float ali_s = 0.f;  // see plain_iteration; set where a stretch begins (wave-uniform)
+  bf16_t ali_s_hi = (bf16_t)0.f, ali_s_lo = (bf16_t)0.f;
   auto plain_iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
     constexpr int PAR = decltype(parity)::value;
     constexpr int PF = TIGHT ? 2 : 3;  // these variants have four registers less to spare
@@ -686,7 +735,19 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const char* kt = s_k[(PAR + 1) & 3];
     const unsigned vt = PAR * TILE_BYTES;
     update_reference(cur_mx);
-    const float neg_m = -m_run;  // finite: the current tile has unmasked scores
+    float neg_m = -m_run;  // finite: the current tile has unmasked scores
+    bool gate_nxt = true;
+    if (GENERAL && seg_on) {
+      // documents: tile i and tile i + 1 have one segment id each; a lane whose query row carries
+      // another id takes no part in the tile - its probabilities are exp2(-inf) = 0 and its row
+      // maximum is -inf.  The ids travel in scalar registers, fetched one tile ahead.
+      const int my_id = s_stash[0][tid];
+      neg_m = (my_id == doc_cur) ? -m_run : RA_NEG_INF;
+      gate_nxt = my_id == doc_nxt;
+      doc_cur = doc_nxt;
+      doc_nxt = doc_far;                                                // requested one iteration ago
+      doc_far = doc_ids[(long long)(tile_base + i + 3) * kKeyTile];    // tile i + 3 exists
+    }
     const unsigned v_dst = v_dst0 + (late_half ? ((PAR + 3) & 3) : ((PAR + 2) & 3)) * TILE_BYTES;
     // ---- S(i+1) MFMAs, then O += P(i) V_i, with the softmax arithmetic of tile i and the row
     // maximum of S(i+1) in their shadow.  The chain of a pair of scores (scale and shift, exp2,
@@ -727,8 +788,16 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       pw[w >> 2][w & 3] = pk[w];
     };
     auto link4 = [&](int w) {
-      lp_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lp_run, false);
-      asm volatile("" : "+v"(lp_run));
+      if constexpr (GENERAL) {
+        // both sums: under ALiBi or inside a short document a row's weight sits on a few keys,
+        // and the rounding of those few terms alone would move the logsumexp by up to 2e-3
+        lr_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lr_run, false);
+        l_run += e[w][0] + e[w][1];
+        asm volatile("" : "+v"(lr_run), "+v"(l_run));
+      } else {
+        lp_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lp_run, false);
+        asm volatile("" : "+v"(lp_run));
+      }
     };
     auto links_of_slot = [&](int gs) {
 #pragma unroll
@@ -741,21 +810,49 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     };
     {
       bf16x8 fr[NOPA];
+      if (GENERAL && alibi_on) {
+        // ALiBi of tile i+1 through the matrix unit: the accumulators start from
+        //   [j, j, 1, 1] x [s_hi, s_lo, c_hi, c_lo] = s j + c = -slope |q_pos - kv_pos| / scale2
+        // with s = +-slope / scale2 (the sign of the stretch), j the key's index in the tile and
+        // c = -s (q_pos - position of the tile's first key), both split into two bf16 words, so
+        // that the score chain below needs no instruction for the bias.  Where the bias is
+        // large the split's error (2^-17 relative) is too, but there the probability is nil.
+        // (recomputed per tile from the lane number: the loop has no register to carry it in)
+        const int ramp_lane = tid & 63;
+        const int rel_i = q_off + q0 + (tid >> 6) * 32 + (ramp_lane & 31) - (kv_off + (tile_base + i + 1) * kKeyTile);
+        const float ali_c = -ali_s * (float)rel_i;
+        const bf16_t c_hi = (bf16_t)ali_c;
+        const bf16_t c_lo = (bf16_t)(ali_c - (float)c_hi);
+        bf16x8 bq;
+        bq[0] = ali_s_hi;
+        bq[1] = ali_s_lo;
+        bq[2] = c_hi;
+        bq[3] = c_lo;
+        bq[4] = bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
+        f32x16 z;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        SN[0][r] = 0.f;
-        SN[1][r] = 0.f;
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        SN[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[0][ramp_lane], bq, z, 0, 0, 0);
+        SN[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[1][ramp_lane], bq, z, 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          SN[0][r] = 0.f;
+          SN[1][r] = 0.f;
+        }
       }
 #pragma unroll
       for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
       bf16x8 q0 = qf[0];
       if (TIGHT) q0 = s_q0[tid];
+      bf16x8 q1 = qf[1];
+      if (GENERAL) q1 = s_q1[tid];
       links_of_slot(-1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int op = 0; op < NOPA; ++op) {
         if (op + PF < NOPA) fr[op + PF] = s_op_frag(kt, op + PF);
-        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? q0 : qf[op >> 1], SN[op & 1], 0, 0, 0);
+        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? q0 : (op < 4 ? q1 : qf[op >> 1]), SN[op & 1], 0, 0, 0);
         if (op == NOPA / 4) global_to_lds16_s(k_run, k_voff[0], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES);
         if (NLD == 2 && op == NOPA * 3 / 4)
           global_to_lds16_s(k_run + k_part, k_voff[NLD - 1], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES + RPI * (D * 2));
@@ -790,6 +887,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         __builtin_amdgcn_sched_barrier(0);
       }
       cur_mx = half_max(fmaxf(mx0, mx1)) * a.scale2;
+      if (GENERAL && seg_on) cur_mx = gate_nxt ? cur_mx : RA_NEG_INF;
     }
     v_run += (long long)kKeyTile * a.v.sl;
   };
@@ -799,27 +897,63 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     request_v(2, 0);  // what the second half of iteration -1 would have requested
     request_v(2, 1);
   }
-  // Three loops over the same sequence of tiles: generic iterations up to the plain stretch, the
-  // plain stretch in whole groups of four, generic iterations for the rest.  Every wave runs n
-  // iterations in total, so the barrier counts agree.
+  // The same sequence of tiles in pieces: generic iterations up to a plain stretch, the stretch in
+  // whole groups of four, ... , generic iterations for the rest.  Every wave runs n iterations in
+  // total, so the barrier counts agree.
   using P0 = std::integral_constant<int, 0>;
   using P1 = std::integral_constant<int, 1>;
   using P2 = std::integral_constant<int, 2>;
   using P3 = std::integral_constant<int, 3>;
-  // iteration i is plain for plain_lo <= i < plain_end
-  const int plain_end =
-      __builtin_amdgcn_readfirstlane(plain_hi - plain_lo < kPlainMinTiles
-                                         ? 0
-                                         : min(min(plain_hi - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));
   int i = 0;
-  for (; i < n && !(i >= plain_lo && i + 4 <= plain_end); i += 4) {
-    iteration(P0{}, i, sa, sb);
-    if (i + 1 < n) iteration(P1{}, i + 1, sb, sa);
-    if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
-    if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
-  }
-  if (i + 4 <= plain_end) {
+  if constexpr (!GENERAL) {
+    // one stretch; iteration i is plain for st_lo[0] <= i < plain_end
+    const int plain_end =
+        __builtin_amdgcn_readfirstlane(st_hi[0] - st_lo[0] < kPlainMinTiles
+                                           ? 0
+                                           : min(min(st_hi[0] - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));
+    for (; i < n && !(i >= st_lo[0] && i + 4 <= plain_end); i += 4) {
+      iteration(P0{}, i, sa, sb);
+      if (i + 1 < n) iteration(P1{}, i + 1, sb, sa);
+      if (i + 2 < n) iteration(P2{}, i + 2, sa, sb);
+      if (i + 3 < n) iteration(P3{}, i + 3, sb, sa);
+    }
+    if (i + 4 <= plain_end) {
+      seek_plain(i);
+      for (; i + 4 <= plain_end; i += 4) {
+        plain_iteration(P0{}, i, sa, sb);
+        plain_iteration(P1{}, i + 1, sb, sa);
+        plain_iteration(P2{}, i + 2, sa, sb);
+        plain_iteration(P3{}, i + 3, sb, sa);
+      }
+    }
+  } else {
+#pragma unroll 1
+  for (int st = 0; st < NST; ++st) {
+    // iteration i is plain for p_lo <= i < p_end
+    const int p_lo = st ? st_lo[1] : st_lo[0], p_hi = st ? st_hi[1] : st_hi[0];
+    const int p_end = __builtin_amdgcn_readfirstlane(
+        min(min(p_hi - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));  // exact sums: no minimum length
+    const int start = max(i, (p_lo + 3) & ~3);  // i is a multiple of four here
+    if (start + 4 > p_end) continue;
+    for (; i < start; i += 4) {
+      iteration(P0{}, i, sa, sb);
+      iteration(P1{}, i + 1, sb, sa);
+      iteration(P2{}, i + 2, sa, sb);
+      iteration(P3{}, i + 3, sb, sa);
+    }
     seek_plain(i);
+    if (GENERAL && seg_on) {
+      doc_cur = doc_ids[(long long)(tile_base + i) * kKeyTile];
+      doc_nxt = doc_ids[(long long)(tile_base + i + 1) * kKeyTile];
+      doc_far = doc_ids[(long long)(tile_base + i + 2) * kKeyTile];
+    }
+    if (GENERAL && alibi_on) {
+      // the first iteration of the stretch computes the scores of tile i + 1
+      ali_s = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
+          __builtin_bit_cast(int, (st ? -slope2 : slope2) / a.scale2)));  // one slope per head
+      ali_s_hi = (bf16_t)ali_s;
+      ali_s_lo = (bf16_t)(ali_s - (float)ali_s_hi);
+    }
     // per-lane values that only the generic iterations use wait in LDS while the plain loop runs:
     // it has no register to spare
     if (GENERAL) {
@@ -828,7 +962,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       s_stash[2][tid] = __float_as_int(slope2);
       seg_r = pre_r = 0;  // already stored
     }
-    for (; i + 4 <= plain_end; i += 4) {
+    for (; i + 4 <= p_end; i += 4) {
       plain_iteration(P0{}, i, sa, sb);
       plain_iteration(P1{}, i + 1, sb, sa);
       plain_iteration(P2{}, i + 2, sa, sb);
@@ -838,6 +972,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       q_seg = s_stash[0][tid];
       q_pre = s_stash[1][tid];
       slope2 = __int_as_float(s_stash[2][tid]);
+    }
+    if (GENERAL && seg_on) {
+      // the scores of tile i, which the next generic iteration turns into probabilities, came
+      // out of the stretch without a mask: rows of another document drop out here
+      if (q_seg != doc_cur) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sa[0][r] = sa[1][r] = RA_NEG_INF;
+      }
     }
     // the plain iterations requested K tiles i .. i+2 without their ids: fetch them for the
     // iterations that follow (the barrier at the top of iteration i publishes them)
@@ -851,6 +993,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         }
       }
     }
+  }
   }
   for (; i < n; i += 4) {
     iteration(P0{}, i, sa, sb);
