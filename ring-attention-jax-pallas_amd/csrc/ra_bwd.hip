@@ -258,7 +258,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
         cnt += __popcll(mask);
       }
       int u_lo, u_hi, u_base;
-      uniform_run(s_list, cnt, lane, u_lo, u_hi, u_base);
+      uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
       if (lane == 0) {
         s_red[8] = cnt;
         s_red[9] = u_lo;
@@ -997,7 +997,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         cnt += __popcll(mask);
       }
       int u_lo, u_hi, u_base;
-      uniform_run(s_list, cnt, lane, u_lo, u_hi, u_base);
+      uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
       if (lane == 0) {
         s_red[16] = cnt;
         s_red[17] = u_lo;

@@ -341,19 +341,21 @@ RA_DEV void tile_id_range(const int* ids, int t, int L, int& mn, int& mx) {
 }
 
 // Executed by ONE wave.  `list` holds `cnt` entries (tile index in bits 0..14, bit 15 set when
-// the tile needs the elementwise segment test).  Finds the first run of entries that need no test
-// and whose tile indices are consecutive: ordinals [start, end), and `tile_base` such that entry
-// i of the run is tile `tile_base + i`.  Such a run can be walked with running addresses.
-RA_DEV void uniform_run(const unsigned short* list, int cnt, int lane, int& start, int& end, int& tile_base) {
+// the tile needs the elementwise segment test).  Finds the first run, at or after ordinal `from`,
+// of entries that need no test and whose tile indices are consecutive: ordinals [start, end), and
+// `tile_base` such that entry i of the run is tile `tile_base + i`.  Such a run can be walked with
+// running addresses.  No run: start = end = cnt.
+RA_DEV void uniform_run(const unsigned short* list, int cnt, int lane, int from, int& start, int& end, int& tile_base) {
   start = -1;
-  for (int base = 0; base < cnt && start < 0; base += 64) {
+  for (int base = from; base < cnt && start < 0; base += 64) {
     const int i = base + lane;
     const bool ok = i < cnt && !(list[i] >> 15);
     const unsigned long long mask = __ballot(ok);
     if (mask) start = base + __ffsll((long long)mask) - 1;
   }
   if (start < 0) {
-    start = end = tile_base = 0;
+    start = end = cnt;
+    tile_base = 0;
     return;
   }
   end = cnt;

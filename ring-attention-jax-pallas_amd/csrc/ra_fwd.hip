@@ -38,7 +38,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   __shared__ __attribute__((aligned(16))) int s_pre[4][kKeyTile];
   __shared__ unsigned short s_list[GENERAL ? kMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
-  __shared__ int s_red[24];
+  __shared__ int s_red[28];
+  __shared__ int s_st[GENERAL ? 8 : 1][12];  // per wave and stretch: first iteration, end, tile_base
   __shared__ int s_stash[GENERAL ? 3 : 1][GENERAL ? kFwdThreads : 1];
   // The GENERAL and MULTI variants are a few registers short in their straight-line loop: the
   // first operand fragment of Q waits here and is fetched once per iteration instead.
@@ -183,6 +184,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // belongs to the tile's document or it does not.  wg_one_doc: all queries of the workgroup
   // share one id, so that a listed tile with one id needs no test at all.
   int run_lo = 0, run_hi = n_act, tile_base = j_lo;
+  // ... and a second such run further on (a workgroup whose queries straddle a document boundary
+  // lists the tiles of both documents, with the tile that holds the boundary between them)
+  int run2_lo = 0, run2_hi = 0, tile_base2 = 0;
   bool wg_one_doc = true;
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     // segment-id range of the workgroup's queries, then one thread per key tile decides
@@ -219,13 +223,17 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         if (f) s_list[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)((j_lo + i) | ((f & 2) << 14));
         cnt += __popcll(mask);
       }
-      int u_lo, u_hi, u_base;
-      uniform_run(s_list, cnt, lane, u_lo, u_hi, u_base);
+      int u_lo, u_hi, u_base, w_lo, w_hi, w_base;
+      uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
+      uniform_run(s_list, cnt, lane, u_hi, w_lo, w_hi, w_base);
       if (lane == 0) {
         s_red[16] = cnt;
         s_red[17] = u_lo;
         s_red[18] = u_hi;
         s_red[19] = u_base;
+        s_red[20] = w_lo;
+        s_red[21] = w_hi;
+        s_red[22] = w_base;
       }
     }
     __syncthreads();
@@ -233,6 +241,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     run_lo = s_red[17];
     run_hi = s_red[18];
     tile_base = s_red[19];
+    run2_lo = s_red[20];
+    run2_hi = s_red[21];
+    tile_base2 = s_red[22];
   }
 
   const bf16_t* kbase = k_ptr + b * a.k.sb + h * a.k.sh;
@@ -313,6 +324,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
   run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
   tile_base = __builtin_amdgcn_readfirstlane(tile_base);
+  run2_lo = __builtin_amdgcn_readfirstlane(run2_lo);
+  run2_hi = __builtin_amdgcn_readfirstlane(min(run2_hi, n));
+  tile_base2 = __builtin_amdgcn_readfirstlane(tile_base2);
   int sb_unused;
   // part t of the request for K tile ordinal j / V tile ordinal j (nothing if the tile does not exist)
   auto request_k = [&](int j, int t) {
@@ -516,9 +530,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // they take the straight-line path without any per-tile classification.  Under ALiBi a stretch
   // must also lie on one side of the diagonal, where -slope |q_pos - kv_pos| is linear in both
   // positions (stretch 0: keys before the wave's queries, stretch 1: keys after them).
-  constexpr int NST = 2;
+  // Stretches 0 and 1 lie in the first run of tiles, 2 and 3 in the second one.
+  constexpr int NST = 4;
   const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
-  int st_lo[2] = {0, 0}, st_hi[2] = {0, 0};
+  int st_lo[NST] = {0, 0, 0, 0}, st_hi[NST] = {0, 0, 0, 0};
   if (wave_on && !(GENERAL && (flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;  // tile indices
     key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kKeyTile,
@@ -534,12 +549,28 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     st_hi[0] = max(min(hi1 - tile_base, run_hi), st_lo[0]);
     st_lo[1] = max(max(lo2 - tile_base, run_lo), st_hi[0]);
     st_hi[1] = max(min(hi - tile_base, run_hi), st_lo[1]);
+    if (GENERAL) {
+      st_lo[2] = max(max(lo - tile_base2, run2_lo), st_hi[1]);
+      st_hi[2] = max(min(hi1 - tile_base2, run2_hi), st_lo[2]);
+      st_lo[3] = max(max(lo2 - tile_base2, run2_lo), st_hi[2]);
+      st_hi[3] = max(min(hi - tile_base2, run2_hi), st_lo[3]);
+    }
   }
+  if constexpr (GENERAL) {
+    // The stretches of this wave wait in LDS (the loops have no scalar register to spare):
+    // iteration i is plain for p_lo <= i < p_end; exact row sums, so no minimum length.
+    if (lane == 0) {
 #pragma unroll
-  for (int st = 0; st < 2; ++st) {  // wave-uniform; now the compiler knows
-    st_lo[st] = __builtin_amdgcn_readfirstlane(st_lo[st]);
-    st_hi[st] = __builtin_amdgcn_readfirstlane(st_hi[st]);
+      for (int st = 0; st < NST; ++st) {
+        const int base = st < 2 ? tile_base : tile_base2, r_hi = st < 2 ? run_hi : run2_hi;
+        s_st[wave][3 * st] = st_lo[st];
+        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, r_hi - 3), a.Lk / kKeyTile - base - 3);
+        s_st[wave][3 * st + 2] = base;
+      }
+    }
   }
+  st_lo[0] = __builtin_amdgcn_readfirstlane(st_lo[0]);  // wave-uniform; now the compiler knows
+  st_hi[0] = __builtin_amdgcn_readfirstlane(st_hi[0]);
 
   // Barrier number k and the requests that follow it (see the loop description above).
   const bool late_half = wave_u >= 4;
@@ -930,9 +961,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 #pragma unroll 1
   for (int st = 0; st < NST; ++st) {
     // iteration i is plain for p_lo <= i < p_end
-    const int p_lo = st ? st_lo[1] : st_lo[0], p_hi = st ? st_hi[1] : st_hi[0];
-    const int p_end = __builtin_amdgcn_readfirstlane(
-        min(min(p_hi - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));  // exact sums: no minimum length
+    const int p_lo = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st]);
+    const int p_end = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st + 1]);
+    tile_base = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st + 2]);
     const int start = max(i, (p_lo + 3) & ~3);  // i is a multiple of four here
     if (start + 4 > p_end) continue;
     for (; i < start; i += 4) {
@@ -950,7 +981,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (GENERAL && alibi_on) {
       // the first iteration of the stretch computes the scores of tile i + 1
       ali_s = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
-          __builtin_bit_cast(int, (st ? -slope2 : slope2) / a.scale2)));  // one slope per head
+          __builtin_bit_cast(int, ((st & 1) ? -slope2 : slope2) / a.scale2)));  // one slope per head
       ali_s_hi = (bf16_t)ali_s;
       ali_s_lo = (bf16_t)(ali_s - (float)ali_s_hi);
     }
