@@ -92,7 +92,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   __shared__ __attribute__((aligned(16))) char s_stat[NB][STAT_BYTES];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
-  __shared__ int s_red[12];
+  __shared__ int s_red[16];
+  // GENERAL: per wave and stretch of straight-line iterations: first tile ordinal, end, tile base
+  __shared__ int s_st[GENERAL ? 4 : 1][12];
+  // A operand of the matrix instruction that adds the ALiBi term to a fresh score tile
+  __shared__ __attribute__((aligned(16))) bf16x8 s_ramp[GENERAL ? 64 : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -163,6 +167,22 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   auto mfma_scores = [&](f32x16& acc, const bf16x8& av, const u32x4& b_acc) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "a"(b_acc));
   };
+  // the same with B in vector registers
+  auto mfma_scores_v = [&](f32x16& acc, const bf16x8& av, const bf16x8& bv) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "v"(bv));
+  };
+  if (GENERAL && tid < 64) {
+    // row l32 of the 32 x 16 operand is [i, i, 1, 1, 0 ...] with i = l32 the query's index in the
+    // tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
+    bf16x8 rf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) rf[e] = (bf16_t)0.f;
+    if (g == 0) {
+      rf[0] = rf[1] = (bf16_t)(float)l32;
+      rf[2] = rf[3] = (bf16_t)1.0f;
+    }
+    s_ramp[tid] = rf;
+  }
   float slope2 = 0.f;
   const float res = a.scale_res, inv_res = 1.0f / a.scale_res;
   if (GENERAL && (flags & RA_BIAS_ALIBI)) slope2 = bs.slopes[h] * kLog2e * inv_res;
@@ -218,8 +238,16 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   query_tile_range(flags, bs.window, kv_off + k0, kv_off + k_hi, q_off, ntiles, kQTile, i_lo, i_hi);
   int n_act = i_hi - i_lo;
   bool use_list = false;
-  // ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` that need no segment test
+  // Ordinals [run_lo, run_hi) are consecutive tiles `tile_base + ordinal` with one segment id
+  // each: inside a straight-line stretch a lane decides per tile whether its key belongs to the
+  // tile's document.  [run2_lo, run2_hi): a second such run behind the first one (a workgroup
+  // that straddles a document boundary has one per document).  wg_one_doc: all keys of the
+  // workgroup carry one id, so one-id tiles need no test in the generic iterations either.
   int run_lo = 0, run_hi = n_act, tile_base = i_lo;
+  int run2_lo = 0, run2_hi = 0, tile_base2 = 0;
+  bool wg_one_doc = true;
+  const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
+  const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     use_list = true;
     int smin = 0x7fffffff, smax = (int)0x80000000;
@@ -244,9 +272,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       int qmin, qmax;
       tile_id_range<kQTile>(q_seg, i, a.Lq, qmin, qmax);
       const bool act = !(qmax < kmin || qmin > kmax);
-      const bool uniform = (kmin == kmax) && (qmin == qmax) && (kmin == qmin);
-      s_flag[i - i_lo] = act ? (uniform ? 1 : 3) : 0;
+      s_flag[i - i_lo] = act ? ((qmin == qmax) ? 1 : 3) : 0;
     }
+    wg_one_doc = kmin == kmax;
     __syncthreads();
     if (wave == 0) {
       int cnt = 0;
@@ -257,13 +285,17 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
         if (f) s_list[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)((i_lo + i) | ((f & 2) << 14));
         cnt += __popcll(mask);
       }
-      int u_lo, u_hi, u_base;
+      int u_lo, u_hi, u_base, w_lo, w_hi, w_base;
       uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
+      uniform_run(s_list, cnt, lane, u_hi, w_lo, w_hi, w_base);
       if (lane == 0) {
         s_red[8] = cnt;
         s_red[9] = u_lo;
         s_red[10] = u_hi;
         s_red[11] = u_base;
+        s_red[12] = w_lo;
+        s_red[13] = w_hi;
+        s_red[14] = w_base;
       }
     }
     __syncthreads();
@@ -271,6 +303,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     run_lo = s_red[9];
     run_hi = s_red[10];
     tile_base = s_red[11];
+    run2_lo = s_red[12];
+    run2_hi = s_red[13];
+    tile_base2 = s_red[14];
   }
   const int n = __builtin_amdgcn_readfirstlane(n_act);
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
@@ -280,7 +315,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
       int e = s_list[i];
-      segbit = e >> 15;
+      segbit = (e >> 15) | (wg_one_doc ? 0 : 1);  // a tile of several ids, or keys of several
       return e & 0x7fff;
     }
     segbit = 0;
@@ -488,8 +523,45 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
 
   // Ordinals [plain_lo, plain_hi) of the query tiles this wave's keys see completely, unmasked
   // and in range: they take the fused path without any per-tile classification.
+  // The per-tile-term variants have up to four such stretches (their bounds wait in LDS): under
+  // ALiBi a stretch must lie on one side of the diagonal, where -slope |q_pos - kv_pos| is linear
+  // in both positions (stretches 0 and 2: queries before the workgroup's keys, 1 and 3: queries
+  // after them); stretches 0 and 1 lie in the first run of one-id tiles, 2 and 3 in the second.
   int plain_lo = 0, plain_hi = 0;
-  if (wave_on && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
+  if constexpr (GENERAL) {
+    int st_lo[4] = {0, 0, 0, 0}, st_hi[4] = {0, 0, 0, 0};
+    if (wave_on && !(flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE))) {
+      int lo, hi;
+      query_tile_plain_range(flags, bs.window, kv_off + kw, kv_off + kw + 31, q_off, a.Lq / kQTile,
+                             kQTile, lo, hi);
+      int lo2 = hi, hi1 = hi;
+      if (alibi_on) {
+        // the same bounds for all waves (the workgroup's first and last key): the waves meet at a
+        // barrier per tile, so a generic iteration in one of them holds up all
+        hi1 = min(hi, floor_div(kv_off + k0 - q_off - (kQTile - 1), kQTile) + 1);     // last query <= first key
+        lo2 = max(lo, ceil_div(kv_off + k0 + KEYS_WG - 1 - q_off, kQTile));          // first query >= last key
+      }
+      const int r2_hi = min(run2_hi, n);
+      st_lo[0] = max(lo - tile_base, run_lo);
+      st_hi[0] = max(min(hi1 - tile_base, run_hi), st_lo[0]);
+      st_lo[1] = max(max(lo2 - tile_base, run_lo), st_hi[0]);
+      st_hi[1] = max(min(hi - tile_base, run_hi), st_lo[1]);
+      st_lo[2] = max(max(lo - tile_base2, run2_lo), st_hi[1]);
+      st_hi[2] = max(min(hi1 - tile_base2, r2_hi), st_lo[2]);
+      st_lo[3] = max(max(lo2 - tile_base2, run2_lo), st_hi[2]);
+      st_hi[3] = max(min(hi - tile_base2, r2_hi), st_lo[3]);
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const int base = st < 2 ? tile_base : tile_base2, r_hi = st < 2 ? run_hi : min(run2_hi, n);
+        // iteration i is plain for first < i < end (tile i+3 must exist, belong to the run and be complete)
+        s_st[wave][3 * st] = st_lo[st];
+        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, r_hi - 3), a.Lq / kQTile - base - 3);
+        s_st[wave][3 * st + 2] = base;
+      }
+    }
+  } else if (wave_on) {
     int lo, hi;
     query_tile_plain_range(flags, bs.window, kv_off + kw, kv_off + kw + 31, q_off, a.Lq / kQTile,
                            kQTile, lo, hi);
@@ -598,9 +670,26 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
 
   // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
   // exists and is complete, so there is nothing to classify and no flag to consult.
+  // The segment ids of a stretch's tiles (one id per tile) travel in scalar registers, fetched
+  // ahead through the constant address space: the compiler uses the scalar cache and tracks the
+  // load in flight itself (the array is not written while the kernel runs).
+  typedef const __attribute__((address_space(4))) int* const_ids;
+  const const_ids doc_ids = (const_ids)(uintptr_t)q_seg;
+  int doc_cur = 0, doc_nxt = 0, doc_far = 0;  // segment ids of tiles i, i + 1, i + 2 of a stretch
+  float ali_s = 0.f;                          // +-slope in score units, set where a stretch begins
+  bf16_t ali_s_hi = (bf16_t)0.f, ali_s_lo = (bf16_t)0.f;
   auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
     constexpr int PHP = (PH + NB - 1) % NB, PH1 = (PH + 1) % NB, PH2 = (PH + 2) % NB, PH3 = (PH + 3) % NB;
+    // documents: a lane whose key carries another id than tile i takes no part in it - its
+    // probabilities are exp2(-inf) = 0
+    float gate = 0.f;
+    if (GENERAL && seg_on) {
+      gate = (k_seg == doc_cur) ? 0.f : RA_NEG_INF;
+      doc_cur = doc_nxt;
+      doc_nxt = doc_far;                                                  // requested one iteration ago
+      doc_far = doc_ids[(long long)(tile_base + i + 3) * kQTile];        // tile i + 3 exists
+    }
     const char* qp = s_q[PHP];
     const char* dop = s_do[PHP];
     const char* qn = s_q[PH1];
@@ -670,6 +759,25 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     // an element (exp2, product, packing) spread over consecutive slots
     float pe[16], de[16];
     constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+    if (GENERAL && alibi_on) {
+      // ALiBi of tile i+1 through the matrix unit: the score accumulators receive
+      //   [r, r, 1, 1] x [s_hi, s_lo, c_hi, c_lo] = s r + c = -slope |q_pos - kv_pos| (score units)
+      // with s = +-slope (the sign of the stretch), r the query's index in the tile and
+      // c = s (position of the tile's first query - kv_pos), both split into two bf16 words, so
+      // that the chain below needs no instruction for the bias.  Where the bias is large the
+      // split's error (2^-17 relative) is too, but there the probability is nil.
+      const int rel_t = q_off + (tile_base + i + 1) * kQTile - (kv_off + kw + l32);
+      const float ali_c = ali_s * (float)rel_t;
+      const bf16_t c_hi = (bf16_t)ali_c;
+      const bf16_t c_lo = (bf16_t)(ali_c - (float)c_hi);
+      bf16x8 bq;
+      bq[0] = ali_s_hi;
+      bq[1] = ali_s_lo;
+      bq[2] = c_hi;
+      bq[3] = c_lo;
+      bq[4] = bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
+      mfma_scores_v(SN, s_ramp[lane], bq);
+    }
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PFN < 2 * KS) fra[op + PFN] = nat_frag(((op + PFN) & 1) ? don : qn, (op + PFN) >> 1);
@@ -684,7 +792,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       for (int e = 0; e < EPO; ++e) {
         const int r = op * EPO + e;
         if (r < 16) {
-          pe[r] = fast_exp2(SC[r] * res);
+          if (GENERAL) pe[r] = fast_exp2(fmaf(SC[r], res, gate));
+          else pe[r] = fast_exp2(SC[r] * res);
           asm volatile("" : "+v"(pe[r]));
         }
         if (r >= 1 && r <= 16) {
@@ -714,10 +823,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   using P3 = std::integral_constant<int, 3>;
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
+  int i = 0;
+  if constexpr (!GENERAL) {
   // iteration i is plain for plain_lo < i < plain_end (tile i+3 must exist and be complete)
   const int plain_end = __builtin_amdgcn_readfirstlane(
-      DENSE ? -1 : min(min(plain_hi - 1, run_hi - 3), a.Lq / kQTile - tile_base - 3));
-  int i = 0;
+      min(min(plain_hi - 1, run_hi - 3), a.Lq / kQTile - tile_base - 3));
   for (; i < n && !(i > plain_lo && i + NB <= plain_end); i += NB) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
     if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
@@ -726,9 +836,47 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
-    if (i + NB <= plain_end) seek_plain(tile_base + i + 3);
-    for (; i + NB <= plain_end; i += NB) {
+  if (i + NB <= plain_end) seek_plain(tile_base + i + 3);
+  for (; i + NB <= plain_end; i += NB) {
+    plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
+    plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+    plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+    plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+    plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+    plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+  }
+  } else if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+#pragma unroll 1
+  for (int st = 0; st < 4; ++st) {
+    // iteration i is plain for p_lo < i < p_end
+    const int p_lo = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st]);
+    const int p_end = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st + 1]);
+    const int start = max(i, ((p_lo + NB) / NB) * NB);  // i is a multiple of six here
+    if (start + NB > p_end) continue;
+    tile_base = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st + 2]);
+    for (; i < start; i += NB) {
+      iteration(P0{}, i, s_a, p_a, s_b, p_b);
+      iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+      iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+      iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+      iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+      iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+    }
+    seek_plain(tile_base + i + 3);
+    if (seg_on) {
+      doc_cur = doc_ids[(long long)(tile_base + i) * kQTile];
+      doc_nxt = doc_ids[(long long)(tile_base + i + 1) * kQTile];
+      doc_far = doc_ids[(long long)(tile_base + i + 2) * kQTile];
+    }
+    if (alibi_on) {
+      // queries before the keys (even stretches): bias = slope (q_pos - kv_pos), rising with the
+      // query's index; queries after them: falling
+      ali_s = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
+          __builtin_bit_cast(int, (st & 1) ? -slope2 : slope2)));  // one slope per head
+      ali_s_hi = (bf16_t)ali_s;
+      ali_s_lo = (bf16_t)(ali_s - (float)ali_s_hi);
+    }
+    for (; i + NB <= p_end; i += NB) {
       plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
       plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
       plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
@@ -736,6 +884,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
       plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
     }
+    if (seg_on && k_seg != doc_cur) {
+      // the scores of tile i, which the next generic iteration turns into probabilities, came
+      // out of the stretch without a mask: keys of another document drop out here
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_a[r] = RA_NEG_INF;
+    }
+  }
   }
   for (; i < n; i += NB) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
@@ -831,14 +986,21 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   __shared__ __attribute__((aligned(16))) int s_pre[NBUF][kDqKeyTile];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
-  __shared__ int s_red[20];
+  __shared__ int s_red[28];
   __shared__ float s_rowc[2][kDqThreads];
+  // GENERAL: per wave and stretch of straight-line iterations: first tile ordinal, end, tile base
+  __shared__ int s_st[GENERAL ? 8 : 1][12];
+  // per-lane values that only the generic iterations use wait here while a stretch runs
+  __shared__ int s_stash[GENERAL ? 3 : 1][GENERAL ? kDqThreads : 1];
+  // A operand of the matrix instruction that writes the ALiBi term into a fresh score tile
+  __shared__ __attribute__((aligned(16))) bf16x8 s_ramp[GENERAL ? 64 : 1];
   // The GENERAL variants are a few registers short in their straight-line loop: the first operand
   // fragments of Q and dO and the per-lane load offsets wait here and are fetched once per
   // iteration instead (a spill to scratch memory would make every iteration wait for all loads).
   constexpr bool TIGHT = GENERAL || MULTI;
   __shared__ __attribute__((aligned(16))) bf16x8 s_q0[TIGHT ? kDqThreads : 1];
   __shared__ __attribute__((aligned(16))) bf16x8 s_do0[TIGHT ? kDqThreads : 1];
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q1[GENERAL ? kDqThreads : 1];
   __shared__ __attribute__((aligned(8))) unsigned s_voff[TIGHT ? kDqThreads : 1][2];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -881,6 +1043,19 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     if (TIGHT) {
       s_q0[tid] = qf[0];
       s_do0[tid] = dof[0];
+    }
+    if (GENERAL) s_q1[tid] = qf[1];
+    if (GENERAL && tid < 64) {
+      // row l32 of the 32 x 16 operand is [j, j, 1, 1, 0 ...] with j = l32 the key's index in the
+      // tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
+      bf16x8 rf;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) rf[e] = (bf16_t)0.f;
+      if (g == 0) {
+        rf[0] = rf[1] = (bf16_t)(float)l32;
+        rf[2] = rf[3] = (bf16_t)1.0f;
+      }
+      s_ramp[tid] = rf;
     }
   }
   const long long row = ((long long)b * a.H + h) * a.Lq + qi_c;
@@ -961,8 +1136,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
                  j_lo, j_hi);
   int n_act = j_hi - j_lo;
   bool use_list = false;
-  // ordinals [run_lo, run_hi) are tiles that need no segment test
-  int run_lo = 0, run_hi = n_act;
+  // Ordinals [run_lo, run_hi) are consecutive tiles `run_base + ordinal` with one segment id
+  // each: inside a straight-line stretch a lane decides per tile whether its query row belongs to
+  // the tile's document.  [run2_lo, run2_hi): a second such run behind the first one (a workgroup
+  // that straddles a document boundary has one per document).  wg_one_doc: all queries of the
+  // workgroup carry one id, so one-id tiles need no test in the generic iterations either.
+  int run_lo = 0, run_hi = n_act, run_base = j_lo;
+  int run2_lo = 0, run2_hi = 0, run2_base = 0;
+  bool wg_one_doc = true;
+  const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     use_list = true;
     int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
@@ -983,9 +1165,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       int kmin, kmax;
       tile_id_range<kDqKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
       const bool act = !(kmax < qmin || kmin > qmax);
-      const bool uniform = (kmin == kmax) && (qmin == qmax) && (kmin == qmin);
-      s_flag[j - j_lo] = act ? (uniform ? 1 : 3) : 0;
+      s_flag[j - j_lo] = act ? ((kmin == kmax) ? 1 : 3) : 0;
     }
+    wg_one_doc = qmin == qmax;
     __syncthreads();
     if (wave == 0) {
       int cnt = 0;
@@ -996,27 +1178,37 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         if (f) s_list[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = (unsigned short)((j_lo + i) | ((f & 2) << 14));
         cnt += __popcll(mask);
       }
-      int u_lo, u_hi, u_base;
+      int u_lo, u_hi, u_base, w_lo, w_hi, w_base;
       uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
+      uniform_run(s_list, cnt, lane, u_hi, w_lo, w_hi, w_base);
       if (lane == 0) {
         s_red[16] = cnt;
         s_red[17] = u_lo;
         s_red[18] = u_hi;
+        s_red[19] = u_base;
+        s_red[20] = w_lo;
+        s_red[21] = w_hi;
+        s_red[22] = w_base;
       }
     }
     __syncthreads();
     n_act = s_red[16];
     run_lo = s_red[17];
     run_hi = s_red[18];
+    run_base = s_red[19];
+    run2_lo = s_red[20];
+    run2_hi = s_red[21];
+    run2_base = s_red[22];
   }
   const int n = __builtin_amdgcn_readfirstlane(n_act);
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
   run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
+  run_base = __builtin_amdgcn_readfirstlane(run_base);
 
   auto tile_at = [&](int i, int& segbit) -> int {
     if (GENERAL && use_list) {
       int e = s_list[i];
-      segbit = e >> 15;
+      segbit = (e >> 15) | (wg_one_doc ? 0 : 1);  // a tile of several ids, or queries of several
       return e & 0x7fff;
     }
     segbit = 0;
@@ -1174,15 +1366,48 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 
   // Ordinals [plain_lo, plain_hi) of the tiles this wave sees completely, unmasked and in
   // range: they take the fused path without any per-tile classification.
+  // The per-tile-term variants have up to four such stretches (their bounds wait in LDS): under
+  // ALiBi a stretch must lie on one side of the diagonal, where -slope |q_pos - kv_pos| is linear
+  // in both positions (stretches 0 and 2: keys before the workgroup's queries, 1 and 3: keys
+  // after them); stretches 0 and 1 lie in the first run of one-id tiles, 2 and 3 in the second.
   int plain_lo = 0, plain_hi = 0;
   // ordinal of tile t inside the run: t - run_tile0
-  int run_tile0 = j_lo;
-  if (run_hi > run_lo) {
-    int sbu;
-    run_tile0 = tile_at(run_lo, sbu) - run_lo;
-  }
-  run_tile0 = __builtin_amdgcn_readfirstlane(run_tile0);
-  if (wave_on && lse_in_range && !(GENERAL && (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
+  int run_tile0 = run_base;
+  const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
+  if constexpr (GENERAL) {
+    int st_lo[4] = {0, 0, 0, 0}, st_hi[4] = {0, 0, 0, 0};
+    if (wave_on && lse_in_range && !(flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE))) {
+      int lo, hi;
+      key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
+                           kDqKeyTile, lo, hi);
+      int lo2 = hi, hi1 = hi;
+      if (alibi_on) {
+        // the same bounds for all waves (the workgroup's first and last query): the waves meet at
+        // a barrier per tile, so a generic iteration in one of them holds up all
+        hi1 = min(hi, floor_div(q_off + q0 - kv_off - (kDqKeyTile - 1), kDqKeyTile) + 1);   // last key <= first query
+        lo2 = max(lo, ceil_div(q_off + q0 + kDqRows - 1 - kv_off, kDqKeyTile));            // first key >= last query
+      }
+      st_lo[0] = max(lo - run_base, run_lo);
+      st_hi[0] = max(min(hi1 - run_base, run_hi), st_lo[0]);
+      st_lo[1] = max(max(lo2 - run_base, run_lo), st_hi[0]);
+      st_hi[1] = max(min(hi - run_base, run_hi), st_lo[1]);
+      const int r2_hi = min(run2_hi, n);
+      st_lo[2] = max(max(lo - run2_base, run2_lo), st_hi[1]);
+      st_hi[2] = max(min(hi1 - run2_base, r2_hi), st_lo[2]);
+      st_lo[3] = max(max(lo2 - run2_base, run2_lo), st_hi[2]);
+      st_hi[3] = max(min(hi - run2_base, r2_hi), st_lo[3]);
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int st = 0; st < 4; ++st) {
+        const int base = st < 2 ? run_base : run2_base, r_hi = st < 2 ? run_hi : min(run2_hi, n);
+        // iteration i is plain for first < i < end (tile i+3 must exist, belong to the run and be complete)
+        s_st[wave][3 * st] = st_lo[st];
+        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, r_hi - 3), a.Lk / kDqKeyTile - base - 3);
+        s_st[wave][3 * st + 2] = base;
+      }
+    }
+  } else if (wave_on && lse_in_range) {
     int lo, hi;
     key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
                          kDqKeyTile, lo, hi);
@@ -1269,7 +1494,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     k_run = kbase + (long long)(tile * kDqKeyTile + RPW * wave_u) * a.k.sl;
     v_run = vbase + (long long)(tile * kDqKeyTile + RPW * wave_u) * a.v.sl;
   };
-  auto issue_run = [&](int buf) {
+  auto issue_run = [&](int buf, int tid) {
     unsigned kvo = k_voff, vvo = v_voff;
     if (TIGHT) {
       kvo = s_voff[tid][0];
@@ -1287,12 +1512,39 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   // exists and is complete, so there is nothing to classify and no flag to consult.  Waves 4..7 take the
   // iteration's barrier between the two MFMA blocks instead of before them (see below).
   const bool late_half = wave_u >= 4;
+  // The segment ids of a stretch's tiles (one id per tile) travel in scalar registers, fetched
+  // ahead through the constant address space: the compiler uses the scalar cache and tracks the
+  // load in flight itself (the array is not written while the kernel runs).
+  typedef const __attribute__((address_space(4))) int* const_ids;
+  const const_ids doc_ids = (const_ids)(uintptr_t)kv_seg;
+  int doc_cur = 0, doc_nxt = 0, doc_far = 0;  // segment ids of tiles i, i + 1, i + 2 of a stretch
+  float ali_s = 0.f;                          // +-slope in score units, set where a stretch begins
+  const int q_first = q0;                     // the workgroup's first query row
+  bf16_t ali_s_hi = (bf16_t)0.f, ali_s_lo = (bf16_t)0.f;
   auto plain_iteration = [&](auto phase, int i, f32x16& SC, f32x16& PC, f32x16& SN, f32x16& PN) {
     constexpr int PH = decltype(phase)::value;
     constexpr int PHP = (PH + NBUF - 1) % NBUF, PH1 = (PH + 1) % NBUF, PH3 = (PH + 3) % NBUF;
     const char* kp = s_k[PHP];
     const char* kn = s_k[PH1];
     const char* vn = s_v[PH1];
+    // The per-tile-term variants rebuild the thread id per iteration (two instructions) instead
+    // of carrying it, or the LDS addresses derived from it, through the loop.
+    int tid_now = tid;
+    if (GENERAL) {
+      int ln;
+      asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(ln));
+      tid_now = wave_u * 64 + ln;
+    }
+    const int tid = tid_now;
+    // documents: a lane whose query row carries another id than tile i takes no part in it - its
+    // probabilities are exp2(-inf) = 0
+    float gate = 0.f;
+    if (GENERAL && seg_on) {
+      gate = (s_stash[0][tid] == doc_cur) ? 0.f : RA_NEG_INF;
+      doc_cur = doc_nxt;
+      doc_nxt = doc_far;                                                      // requested one iteration ago
+      doc_far = doc_ids[(long long)(run_tile0 + i + 3) * kDqKeyTile];        // tile i + 3 exists
+    }
     // operands of the dQ^T product come from tile i-1, visible since two barriers ago
     bf16x8 frb[2 * DB];
 #pragma unroll
@@ -1317,7 +1569,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         fra[o2] = nat_frag((o2 & 1) ? vn : kn, o2 >> 1);
       }
       acc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frb[op], dsf[op / DB], acc[op % DB], 0, 0, 0);
-      if (op == 0) issue_run(PH3);  // next loads: their issue hides behind the MFMAs
+      if (op == 0) issue_run(PH3, tid);  // next loads: their issue hides behind the MFMAs
       __builtin_amdgcn_sched_barrier(0);
     }
     if (late_half) {
@@ -1329,11 +1581,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 #pragma unroll
       for (int op = 0; op < PF; ++op) fra[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
     }
-    bf16x8 q0 = qf[0], do0 = dof[0];
+    bf16x8 q0 = qf[0], do0 = dof[0], q1 = qf[1];
     if (TIGHT) {
       q0 = s_q0[tid];
       do0 = s_do0[tid];
     }
+    if (GENERAL) q1 = s_q1[tid];
     // The chain of a score element (exp2 and the scaled dP, their product, the packing of a
     // pair) is spread over three consecutive MFMA slots, one link per slot, so that no vector
     // instruction waits for the result of the one before it.
@@ -1344,7 +1597,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       for (int e = 0; e < EPO; ++e) {
         const int r = slot * EPO + e;
         if (r >= 0 && r < 16) {
-          ev[r] = fast_exp2(SC[r] * a.scale_res);
+          if (GENERAL) ev[r] = fast_exp2(fmaf(SC[r], a.scale_res, gate));
+          else ev[r] = fast_exp2(SC[r] * a.scale_res);
           uv[r] = fmaf(PC[r], c_row, cd_row);
           asm volatile("" : "+v"(ev[r]), "+v"(uv[r]));  // pins the arithmetic between two MFMAs
         }
@@ -1367,6 +1621,33 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         }
       }
     };
+    if (GENERAL && alibi_on) {
+      // ALiBi of tile i+1 through the matrix unit: the accumulators start from
+      //   [j, j, 1, 1] x [s_hi, s_lo, c_hi, c_lo] = s j + c = -slope |q_pos - kv_pos| (score units)
+      // with s = +-slope (the sign of the stretch), j the key's index in the tile and
+      // c = -s (q_pos - position of the tile's first key), both split into two bf16 words, so
+      // that the chain below needs no instruction for the bias.  Where the bias is large the
+      // split's error (2^-17 relative) is too, but there the probability is nil.
+      // (recomputed per tile from the lane number: the loop has no register to carry it in)
+      const int ramp_lane = tid & 63;
+      const int rel_i = q_off + q_first + (tid >> 6) * 32 + (ramp_lane & 31) - (kv_off + (run_tile0 + i + 1) * kDqKeyTile);
+      const float ali_c = -ali_s * (float)rel_i;
+      const bf16_t c_hi = (bf16_t)ali_c;
+      const bf16_t c_lo = (bf16_t)(ali_c - (float)c_hi);
+      bf16x8 bq;
+      bq[0] = ali_s_hi;
+      bq[1] = ali_s_lo;
+      bq[2] = c_hi;
+      bq[3] = c_lo;
+      bq[4] = bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
+      f32x16 z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[ramp_lane], bq, z, 0, 0, 0);
+    } else if (GENERAL) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) SN[r] = 0.f;
+    }
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PF < 2 * KS) fra[op + PF] = nat_frag(((op + PF) & 1) ? vn : kn, (op + PF) >> 1);
@@ -1375,10 +1656,11 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) z[r] = 0.f;
         if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], do0, z, 0, 0, 0);
+        else if (GENERAL) SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], q0, SN, 0, 0, 0);
         else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], q0, z, 0, 0, 0);
       } else {
         if (op & 1) PN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], dof[op >> 1], PN, 0, 0, 0);
-        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], qf[op >> 1], SN, 0, 0, 0);
+        else SN = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fra[op], op == 2 ? q1 : qf[op >> 1], SN, 0, 0, 0);
       }
       chain_links(op);
       __builtin_amdgcn_sched_barrier(0);
@@ -1396,11 +1678,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   using P3 = std::integral_constant<int, 3>;
   using P4 = std::integral_constant<int, 4>;
   using P5 = std::integral_constant<int, 5>;
+  int i = 0;
+  if constexpr (!GENERAL) {
   // iteration i is plain for plain_lo < i < plain_end
   // (tile i+3 must exist, belong to the run and be complete)
   const int plain_end = __builtin_amdgcn_readfirstlane(
-      DENSE ? -1 : min(min(plain_hi - 1, min(run_hi, n) - 3), a.Lk / kDqKeyTile - run_tile0 - 3));
-  int i = 0;
+      min(min(plain_hi - 1, min(run_hi, n) - 3), a.Lk / kDqKeyTile - run_tile0 - 3));
   for (; i < n && !(i > plain_lo && i + 6 <= plain_end); i += 6) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
     if (i + 1 < n) iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
@@ -1409,10 +1692,9 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     if (i + 4 < n) iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     if (i + 5 < n) iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+  {
     const bool stretch = i + 6 <= plain_end;
     if (stretch) seek_plain(run_tile0 + i + 3);
-    if (GENERAL && stretch) seg_r = pre_r = 0;  // stored already; not carried through the stretch
     if (stretch) {
       // the two row constants of the stretch replace the two of the generic iterations, which
       // wait in LDS meanwhile (the kernel has no register to spare)
@@ -1434,7 +1716,69 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       neg_lse2 = s_rowc[0][tid];
       delta = s_rowc[1][tid];
     }
-    if (GENERAL && stretch && tid < kDqKeyTile) {
+  }
+  } else if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+#pragma unroll 1
+  for (int st = 0; st < 4; ++st) {
+    // iteration i is plain for p_lo < i < p_end
+    const int p_lo = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st]);
+    const int p_end = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st + 1]);
+    const int start = max(i, ((p_lo + 6) / 6) * 6);  // i is a multiple of six here
+    if (start + 6 > p_end) continue;
+    run_tile0 = __builtin_amdgcn_readfirstlane(s_st[wave_u][3 * st + 2]);
+    for (; i < start; i += 6) {
+      iteration(P0{}, i, s_a, p_a, s_b, p_b);
+      iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+      iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+      iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+      iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+      iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+    }
+    seek_plain(run_tile0 + i + 3);
+    if (seg_on) {
+      doc_cur = doc_ids[(long long)(run_tile0 + i) * kDqKeyTile];
+      doc_nxt = doc_ids[(long long)(run_tile0 + i + 1) * kDqKeyTile];
+      doc_far = doc_ids[(long long)(run_tile0 + i + 2) * kDqKeyTile];
+    }
+    if (alibi_on) {
+      // keys before the queries (even stretches): bias = -slope (q_pos - kv_pos), rising with the
+      // key's index; keys after them: falling
+      ali_s = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
+          __builtin_bit_cast(int, (st & 1) ? -slope2 : slope2)));  // one slope per head
+      ali_s_hi = (bf16_t)ali_s;
+      ali_s_lo = (bf16_t)(ali_s - (float)ali_s_hi);
+    }
+    seg_r = pre_r = 0;  // stored already; not carried through the stretch
+    // the two row constants of the stretch replace the two of the generic iterations, which wait
+    // in LDS meanwhile with everything else only the generic iterations use
+    c_row = fast_exp2(neg_lse2);
+    cd_row = -c_row * delta;
+    s_rowc[0][tid] = neg_lse2;
+    s_rowc[1][tid] = delta;
+    neg_lse2 = delta = 0.f;
+    s_stash[0][tid] = q_seg;
+    s_stash[1][tid] = q_pre;
+    s_stash[2][tid] = __float_as_int(slope2);
+    for (; i + 6 <= p_end; i += 6) {
+      plain_iteration(P0{}, i, s_a, p_a, s_b, p_b);
+      plain_iteration(P1{}, i + 1, s_b, p_b, s_a, p_a);
+      plain_iteration(P2{}, i + 2, s_a, p_a, s_b, p_b);
+      plain_iteration(P3{}, i + 3, s_b, p_b, s_a, p_a);
+      plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
+      plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
+    }
+    neg_lse2 = s_rowc[0][tid];
+    delta = s_rowc[1][tid];
+    q_seg = s_stash[0][tid];
+    q_pre = s_stash[1][tid];
+    slope2 = __int_as_float(s_stash[2][tid]);
+    if (seg_on && q_seg != doc_cur) {
+      // the scores of tile i, which the next generic iteration turns into probabilities, came
+      // out of the stretch without a mask: rows of another document drop out here
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_a[r] = RA_NEG_INF;
+    }
+    if (tid < kDqKeyTile) {
       // the stretch moved no ids: those of the two tiles in flight are fetched now (i is a
       // multiple of 6 here: tile i+1 lives in buffer 1, the ids of tile i+2 wait in registers
       // for the top of the next iteration, as after a generic iteration)
@@ -1450,6 +1794,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         if (kv_pre) pre_r = kv_pre[kk];
       }
     }
+  }
   }
   for (; i < n; i += 6) {
     iteration(P0{}, i, s_a, p_a, s_b, p_b);
