@@ -90,9 +90,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   __shared__ __attribute__((aligned(16))) char s_do[NB][TILE_BYTES];
   // per tile and row: -lse * log2(e) / scale_res (-inf for a fully masked row), -delta, segment id, prefix flag
   __shared__ __attribute__((aligned(16))) char s_stat[NB][STAT_BYTES];
+  // the same words as they arrive from memory, one per lane and tile (see store_stat)
+  __shared__ __attribute__((aligned(16))) unsigned s_raw[NB][NT];
   __shared__ unsigned short s_list[GENERAL ? kBwdMaxListTiles : 1];
   __shared__ unsigned char s_flag[GENERAL ? kBwdMaxListTiles : 1];
-  __shared__ int s_red[16];
+  __shared__ int s_red[20];
   // GENERAL: per wave and stretch of straight-line iterations: first tile ordinal, end, tile base
   __shared__ int s_st[GENERAL ? 4 : 1][12];
   // A operand of the matrix instruction that adds the ALiBi term to a fresh score tile
@@ -245,6 +247,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   // workgroup carry one id, so one-id tiles need no test in the generic iterations either.
   int run_lo = 0, run_hi = n_act, tile_base = i_lo;
   int run2_lo = 0, run2_hi = 0, tile_base2 = 0;
+  // the listed tiles count up without a gap from the start of a run to ordinal cons_hi / cons2_hi
+  int cons_hi = n_act, cons2_hi = 0;
   bool wg_one_doc = true;
   const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
   const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
@@ -288,7 +292,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       int u_lo, u_hi, u_base, w_lo, w_hi, w_base;
       uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
       uniform_run(s_list, cnt, lane, u_hi, w_lo, w_hi, w_base);
+      const int c_hi = consecutive_end(s_list, cnt, lane, u_lo);
+      const int c2_hi = consecutive_end(s_list, cnt, lane, w_lo);
       if (lane == 0) {
+        s_red[15] = c_hi;
+        s_red[16] = c2_hi;
         s_red[8] = cnt;
         s_red[9] = u_lo;
         s_red[10] = u_hi;
@@ -306,6 +314,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     run2_lo = s_red[12];
     run2_hi = s_red[13];
     tile_base2 = s_red[14];
+    cons_hi = s_red[15];
+    cons2_hi = s_red[16];
   }
   const int n = __builtin_amdgcn_readfirstlane(n_act);
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
@@ -343,9 +353,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     do_voff[t] = (unsigned)(((long long)(lane / CPR) * a.dout.sl + ld_off[t]) * 2);
   }
   // The per-row words of a tile: lane l of every wave fetches word class (l / 8) % NSTAT of row
-  // 8 * wave + l % 8 into a register (lanes 32..63 repeat lanes 0..31), and writes it, converted,
-  // to s_stat when the tile is awaited.  The load is issued as inline assembly like the tile
-  // loads, so the compiler adds no waits of its own; three registers rotate (tiles i+1 .. i+3).
+  // 8 * wave + l % 8 (lanes 32..63 repeat lanes 0..31) straight into LDS, like the tile itself and
+  // counted with the tile's loads, and moves it, converted, to s_stat when the tile is awaited (a
+  // lane reads only what it fetched itself, so its own load counter is all it needs to watch).
   const int st_class = (lane >> 3) & (NSTAT - 1);
   const int st_row = 8 * wave + (lane & 7);
   const char* st_src;
@@ -360,15 +370,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const unsigned st_dst = (unsigned)(st_class * (kQTile * 4) + st_row * 4);
   const float st_mul = st_class == 0 ? -kLog2e * inv_res : -1.0f;
   const float st_fix = st_class == 0 ? RA_NEG_INF : 0.f;
-  unsigned xr[3] = {0u, 0u, 0u};
-  auto load_stat = [&](const char* p, unsigned& x) {
-    asm volatile("global_load_dword %0, %1, off" : "=v"(x) : "v"(p) : "memory");
+  auto load_stat = [&](const char* p, int buf) {
+    global_to_lds4(p, RA_LDS_ADDR(&s_raw[0][0]) + buf * (NT * 4) + wave_u * 256);
   };
-  auto issue_tile = [&](int it, int buf, unsigned& x) {
+  auto issue_tile = [&](int it, int buf) {
     const int q0 = it * kQTile;
     const unsigned q_dst = RA_LDS_ADDR(&s_q[0][0]) + buf * TILE_BYTES + wave_u * 8 * ROWB;
     const unsigned do_dst = RA_LDS_ADDR(&s_do[0][0]) + buf * TILE_BYTES + wave_u * 8 * ROWB;
-    load_stat(st_src + 4ll * min(q0 + st_row, a.Lq - 1), x);
+    load_stat(st_src + 4ll * min(q0 + st_row, a.Lq - 1), buf);
     if (q0 + kQTile <= a.Lq) {
       // wave-uniform row addresses in scalar registers, per-lane part in one VGPR
       const bf16_t* qs = qbase + (long long)(q0 + 8 * wave_u) * a.q.sl;
@@ -390,8 +399,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     }
   };
   // converts the awaited tile's per-row word and publishes it (the caller has waited for it)
-  auto store_stat = [&](int buf, unsigned& x) {
-    asm volatile("" : "+v"(x));
+  auto store_stat = [&](int buf) {
+    asm volatile("" ::: "memory");  // the read below stays behind the wait for the load
+    const unsigned x = s_raw[buf][tid];
     // lse -> -lse * log2(e), but -inf for a fully masked row (lse = -inf) so that its P is 0;
     // delta -> -delta, but 0 for the NaN that a fully masked output row produces
     float v = __uint_as_float(x) * st_mul;
@@ -512,12 +522,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   // ---- prologue: tiles 0, 1, 2 requested, S(0) and dP(0) computed ------------------------------
   {
     int sbu;
-    if (n > 0) issue_tile(tile_at(0, sbu), 0, xr[0]);
-    if (n > 1) issue_tile(tile_at(1, sbu), 1, xr[1]);
-    if (n > 2) issue_tile(tile_at(2, sbu), 2, xr[2]);  // its statistics are stored in iteration 1
+    if (n > 0) issue_tile(tile_at(0, sbu), 0);
+    if (n > 1) issue_tile(tile_at(1, sbu), 1);
+    if (n > 2) issue_tile(tile_at(2, sbu), 2);  // its statistics are stored in iteration 0
     __builtin_amdgcn_s_waitcnt(0);
-    if (n > 0) store_stat(0, xr[0]);
-    if (n > 1) store_stat(1, xr[1]);
+    if (n > 0) store_stat(0);
+    if (n > 1) store_stat(1);
   }
   __syncthreads();
 
@@ -554,10 +564,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     if (lane == 0) {
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
-        const int base = st < 2 ? tile_base : tile_base2, r_hi = st < 2 ? run_hi : min(run2_hi, n);
-        // iteration i is plain for first < i < end (tile i+3 must exist, belong to the run and be complete)
+        const int base = st < 2 ? tile_base : tile_base2, c_hi = st < 2 ? cons_hi : cons2_hi;
+        // iteration i is plain for first < i < end.  It requests tile i + 3 by running addresses:
+        // where the list goes on that must be the listed tile, behind the list's end it only has
+        // to lie inside the shard (nobody reads it).
+        const int list_end = c_hi >= n ? 0x3fffffff : c_hi - 3;
         s_st[wave][3 * st] = st_lo[st];
-        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, r_hi - 3), a.Lq / kQTile - base - 3);
+        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, list_end), a.Lq / kQTile - base - 3);
         s_st[wave][3 * st + 2] = base;
       }
     }
@@ -606,14 +619,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     // before the tile is read
     if (i + 2 < n) {
       RA_WAIT_VMCNT(LPT - 1);
-      store_stat(PH2, xr[PH2 % 3]);
+      store_stat(PH2);
     } else {
       RA_WAIT_VMCNT(0);
     }
     __syncthreads();
     if (i + 3 < n) {
       int sbu;
-      issue_tile(tile_at(i + 3, sbu), PH3, xr[PH3 % 3]);
+      issue_tile(tile_at(i + 3, sbu), PH3);
     }
     if (pend_valid) {
       bf16x8 pf[2], dsf[2];
@@ -728,7 +741,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       else dv[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pf[ks], frb[op], dv[db], 0, 0, 0);
       // next tile's loads, one instruction group per MFMA: their issue hides behind the MFMAs
       if (op == 0) {
-        load_stat(st_run, xr[PH3 % 3]);
+        load_stat(st_run, PH3);
         st_run += kQTile * 4;
       }
       if (op == 1) {
@@ -786,7 +799,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       if (op == 2) {
         // the per-row word of tile i+2 is the oldest load but those of its tile and of tile i+3
         RA_WAIT_VMCNT(2 * LPT - 1);
-        store_stat(PH2, xr[PH2 % 3]);
+        store_stat(PH2);
       }
 #pragma unroll
       for (int e = 0; e < EPO; ++e) {
@@ -1143,6 +1156,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   // workgroup carry one id, so one-id tiles need no test in the generic iterations either.
   int run_lo = 0, run_hi = n_act, run_base = j_lo;
   int run2_lo = 0, run2_hi = 0, run2_base = 0;
+  // the listed tiles count up without a gap from the start of a run to ordinal cons_hi / cons2_hi
+  int cons_hi = n_act, cons2_hi = 0;
   bool wg_one_doc = true;
   const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
@@ -1181,7 +1196,11 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       int u_lo, u_hi, u_base, w_lo, w_hi, w_base;
       uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
       uniform_run(s_list, cnt, lane, u_hi, w_lo, w_hi, w_base);
+      const int c_hi = consecutive_end(s_list, cnt, lane, u_lo);
+      const int c2_hi = consecutive_end(s_list, cnt, lane, w_lo);
       if (lane == 0) {
+        s_red[23] = c_hi;
+        s_red[24] = c2_hi;
         s_red[16] = cnt;
         s_red[17] = u_lo;
         s_red[18] = u_hi;
@@ -1199,6 +1218,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     run2_lo = s_red[20];
     run2_hi = s_red[21];
     run2_base = s_red[22];
+    cons_hi = s_red[23];
+    cons2_hi = s_red[24];
   }
   const int n = __builtin_amdgcn_readfirstlane(n_act);
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
@@ -1400,10 +1421,13 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     if (lane == 0) {
 #pragma unroll
       for (int st = 0; st < 4; ++st) {
-        const int base = st < 2 ? run_base : run2_base, r_hi = st < 2 ? run_hi : min(run2_hi, n);
-        // iteration i is plain for first < i < end (tile i+3 must exist, belong to the run and be complete)
+        const int base = st < 2 ? run_base : run2_base, c_hi = st < 2 ? cons_hi : cons2_hi;
+        // iteration i is plain for first < i < end.  It requests tile i + 3 by running addresses:
+        // where the list goes on that must be the listed tile, behind the list's end it only has
+        // to lie inside the shard (nobody reads it).
+        const int list_end = c_hi >= n ? 0x3fffffff : c_hi - 3;
         s_st[wave][3 * st] = st_lo[st];
-        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, r_hi - 3), a.Lk / kDqKeyTile - base - 3);
+        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, list_end), a.Lk / kDqKeyTile - base - 3);
         s_st[wave][3 * st + 2] = base;
       }
     }

@@ -157,16 +157,25 @@ struct TileStage {
 // barrier that publishes the tile).  The "x2" form moves two pieces that are 1 KiB apart in
 // LDS with one M0 write: the instruction offset applies to the LDS address AND to the global
 // address, so the second base must already have 1024 bytes subtracted.
+// The compiler inserts no wait states around the instructions of an assembly statement, so the
+// statements carry their own: the LDS address reaches M0 one wait state before the load uses it,
+// and a scalar base address that the compiler may have just restored from a vector register
+// lane (v_readlane: a vector instruction writing a scalar register) is five wait states old
+// before the memory instruction reads it.
 RA_DEV void global_to_lds16(const void* gptr, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
 RA_DEV void global_to_lds16_s(const void* sbase, unsigned voff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory", "m0");
 }
 RA_DEV void global_to_lds16_s_x2(const void* sbase0, unsigned voff0, const void* sbase1_minus_1k, unsigned voff1,
                                  unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %4\n\tglobal_load_lds_dwordx4 %1, %0\n\tglobal_load_lds_dwordx4 %3, %2 offset:1024"
+  asm volatile("s_mov_b32 m0, %4\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %0\n\tglobal_load_lds_dwordx4 %3, %2 offset:1024"
                : : "s"(sbase0), "v"(voff0), "s"(sbase1_minus_1k), "v"(voff1), "s"(lds_addr) : "memory", "m0");
+}
+// one dword per lane: lane l's word lands at lds_addr + 4 l
+RA_DEV void global_to_lds4(const void* gptr, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
 // LDS byte address of an object declared __shared__
 #define RA_LDS_ADDR(obj) ((unsigned)(uintptr_t)(lds_char*)(obj))
@@ -369,6 +378,19 @@ RA_DEV void uniform_run(const unsigned short* list, int cnt, int lane, int from,
     }
   }
   tile_base = (list[start] & 0x7fff) - start;
+}
+
+// Executed by ONE wave.  First ordinal behind `from` whose tile index does not follow its
+// predecessor's (`cnt` if the list counts up to its end): up to there, loads that advance by one
+// tile per iteration fetch exactly the listed tiles.
+RA_DEV int consecutive_end(const unsigned short* list, int cnt, int lane, int from) {
+  for (int base = from; base < cnt; base += 64) {
+    const int i = base + lane;
+    const bool brk = i < cnt && i > from && (list[i] & 0x7fff) != (list[i - 1] & 0x7fff) + 1;
+    const unsigned long long mask = __ballot(brk);
+    if (mask) return base + __ffsll((long long)mask) - 1;
+  }
+  return cnt;
 }
 
 // Decode the flat workgroup id into (batch*head index, tile index).  Workgroups are handed

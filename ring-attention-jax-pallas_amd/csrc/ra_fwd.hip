@@ -187,6 +187,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // ... and a second such run further on (a workgroup whose queries straddle a document boundary
   // lists the tiles of both documents, with the tile that holds the boundary between them)
   int run2_lo = 0, run2_hi = 0, tile_base2 = 0;
+  // the listed tiles count up without a gap from the start of a run to ordinal cons_hi / cons2_hi
+  int cons_hi = n_act, cons2_hi = 0;
   bool wg_one_doc = true;
   if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
     // segment-id range of the workgroup's queries, then one thread per key tile decides
@@ -226,6 +228,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       int u_lo, u_hi, u_base, w_lo, w_hi, w_base;
       uniform_run(s_list, cnt, lane, 0, u_lo, u_hi, u_base);
       uniform_run(s_list, cnt, lane, u_hi, w_lo, w_hi, w_base);
+      const int c_hi = consecutive_end(s_list, cnt, lane, u_lo);
+      const int c2_hi = consecutive_end(s_list, cnt, lane, w_lo);
       if (lane == 0) {
         s_red[16] = cnt;
         s_red[17] = u_lo;
@@ -234,6 +238,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         s_red[20] = w_lo;
         s_red[21] = w_hi;
         s_red[22] = w_base;
+        s_red[23] = c_hi;
+        s_red[24] = c2_hi;
       }
     }
     __syncthreads();
@@ -244,6 +250,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     run2_lo = s_red[20];
     run2_hi = s_red[21];
     tile_base2 = s_red[22];
+    cons_hi = s_red[23];
+    cons2_hi = s_red[24];
   }
 
   const bf16_t* kbase = k_ptr + b * a.k.sb + h * a.k.sh;
@@ -559,12 +567,16 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   if constexpr (GENERAL) {
     // The stretches of this wave wait in LDS (the loops have no scalar register to spare):
     // iteration i is plain for p_lo <= i < p_end; exact row sums, so no minimum length.
+    // Iteration i requests tiles up to i + 3 by running addresses: where the list goes on they
+    // must be the listed ones, behind the list's end they only have to lie inside the shard
+    // (nobody reads them).
     if (lane == 0) {
 #pragma unroll
       for (int st = 0; st < NST; ++st) {
-        const int base = st < 2 ? tile_base : tile_base2, r_hi = st < 2 ? run_hi : run2_hi;
+        const int base = st < 2 ? tile_base : tile_base2, c_hi = st < 2 ? cons_hi : cons2_hi;
+        const int list_end = c_hi >= n ? 0x3fffffff : c_hi - 3;
         s_st[wave][3 * st] = st_lo[st];
-        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, r_hi - 3), a.Lk / kKeyTile - base - 3);
+        s_st[wave][3 * st + 1] = min(min(st_hi[st] - 1, list_end), a.Lk / kKeyTile - base - 3);
         s_st[wave][3 * st + 2] = base;
       }
     }
