@@ -215,6 +215,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const int* q_pre_ptr = bs.q_pre;
   const float* dense_ptr = bs.dense;
   int n_shards = 1;
+  int tiles_listed = 0;  // over all shards of the pass: none, and the workgroup leaves its carry / gradients as they are
   if constexpr (MULTI) n_shards = ring.count[blockIdx.y];
   for (int shard = 0; shard < n_shards; ++shard) {
   if constexpr (MULTI) {
@@ -318,6 +319,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     cons2_hi = s_red[16];
   }
   const int n = __builtin_amdgcn_readfirstlane(n_act);
+  tiles_listed += n;
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
   run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
   tile_base = __builtin_amdgcn_readfirstlane(tile_base);
@@ -924,6 +926,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     compute_dkdv(pf, dsf, s_q[0] + last * TILE_BYTES, s_do[0] + last * TILE_BYTES);
   }
   }  // query shards
+  if (tiles_listed == 0) return;  // nothing to add
   // ---- accumulate into the fp32 gradients owned by this key slab ------------------------------
   // All loads of an array are issued before the first value is needed: a load - add - store chain
   // per element would cost one memory round trip each, a hundred in a row with nothing to hide them.
@@ -1113,6 +1116,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   const int* kv_pre_ptr = bs.kv_pre;
   const float* dense_ptr = bs.dense;
   int n_shards = 1;
+  int tiles_listed = 0;  // over all shards of the pass: none, and the workgroup leaves its carry / gradients as they are
   if constexpr (MULTI) n_shards = ring.count[blockIdx.y];
   for (int shard = 0; shard < n_shards; ++shard) {
   if constexpr (MULTI) {
@@ -1222,6 +1226,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     cons2_hi = s_red[24];
   }
   const int n = __builtin_amdgcn_readfirstlane(n_act);
+  tiles_listed += n;
   run_lo = __builtin_amdgcn_readfirstlane(run_lo);
   run_hi = __builtin_amdgcn_readfirstlane(min(run_hi, n));
   run_base = __builtin_amdgcn_readfirstlane(run_base);
@@ -1835,6 +1840,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     compute_dq(dsf, s_k[0] + ((n - 1) % NBUF) * TILE_BYTES);
   }
   }  // key/value shards
+  if (tiles_listed == 0) return;  // nothing to add
   if (q_valid) {
     float* dq_res = a.dq;
     if constexpr (MULTI) dq_res = ring.x0[blockIdx.y];

@@ -1046,6 +1046,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   }
   if (!late_half) sync(n);  // both halves pass the same number of barriers
   }  // key/value shards
+  // A wave that gathered no probability mass (no tile listed for its workgroup, or every score
+  // masked) has nothing to merge: with l_step = 0 and an unchanged maximum the merge below is the
+  // identity, so the carry's 32 rows stay where they are, unread.
+  if (__all(l_run == 0.f && lr_run == 0.f && lp_run == 0.f)) return;
   // ---- merge this step into the carry ---------------------------------------------------------
   // o = o_in 2^(m_in - m_out) + o_step 2^(m_run - m_out) l_step / lr_step,  l likewise with the
   // exact sum, m_out = exact maximum over carry and step.
