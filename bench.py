@@ -243,8 +243,10 @@ def cpu_baseline(D, config="sample"):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=3)
-    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default: 3 for the 0.5 s steps of C3b / C3a, 20 for the millisecond steps of "
+                         "the small workloads, whose first launches would otherwise dominate the clock)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (default: 1, small workloads 3)")
     ap.add_argument("--workload", default="C3b", choices=sorted(WORKLOADS))
     ap.add_argument("--impl", default="hip", choices=["hip", "hip_fused"],
                     help="hip: one launch per ring step (the headline); hip_fused: one launch per ring pass, "
@@ -282,6 +284,11 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     w = WORKLOADS[args.workload]
+    small = args.workload in ("C2", "C4", "C5")
+    if args.steps is None:
+        args.steps = 20 if small else 3
+    if args.warmup is None:
+        args.warmup = 3 if small else 1
     B, H, D, S, n = w["B"], w["H"], w["D"], w["S"], w["n"]
     L = S // n
     # q, k, v ~ N(0, std^2), dO ~ N(0, 1) from numpy.random.default_rng(0) in fp32, rounded to bf16

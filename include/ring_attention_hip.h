@@ -43,6 +43,7 @@ extern "C" {
 #define RA_ERR_BIAS (-5)        /* inconsistent bias description                    */
 #define RA_ERR_HIP (-6)         /* a HIP runtime call failed (see ra_last_error)    */
 #define RA_ERR_DTYPE (-7)       /* unknown output dtype code                        */
+#define RA_ERR_TOO_LARGE (-8)   /* a whole-ring launch cannot hold these passes     */
 
 /* Bias terms, OR-ed into ra_bias.flags.  They are the device-side form of the reference's
  * bias_fn (ring.py:107,186): each term is evaluated per score tile from token positions
@@ -204,6 +205,30 @@ int ra_bwd_dq_passes(const ra_bwd_step_params* steps, const int32_t* steps_per_p
                      void* stream);
 int ra_bwd_dkdv_passes(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes,
                        void* stream);
+
+/* The WHOLE ring in one launch with nothing in between.  `steps` / `steps_per_pass` as for the
+ * *_passes entry points, but every pass holds ALL the blocks of its resident shard (at least one;
+ * blocks that a positional mask rules out may be listed, they are skipped), so a workgroup
+ * finishes its rows inside the launch and no intermediate state goes through memory:
+ *  - ra_fwd_ring = zero carry (ra_fwd_init) + ra_fwd_passes + ra_fwd_finalize_passes: the carry
+ *    (ring.py:104-132) stays in registers, `out` (bf16 or fp32, pass p at p * out_stride_pass
+ *    elements, strides in elements) and `lse` ([n_passes, B, H, Lq] fp32) receive what
+ *    ring.py:134-137 returns.  The o / m / l fields of the blocks are not used.
+ *  - ra_bwd_dq_ring / ra_bwd_dkdv_ring = zeroed accumulators + ra_bwd_*_passes +
+ *    ra_bwd_finalize_passes: dq (per query shard), dk and dv (per key/value shard, same strides)
+ *    are stored as bf16 (ring.py:208-210).  The dq / dk / dv fields of the blocks are not used.
+ * Result pointers must be aligned to four elements and the strides multiples of four.  Results
+ * agree with the split entry points to rounding (the final division is folded differently), not
+ * bit for bit.  RA_ERR_TOO_LARGE, with nothing launched, when one launch cannot hold the passes
+ * (more than 16 passes, more than 16 distinct travelling shards): use the split entry points. */
+int ra_fwd_ring(const ra_fwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* out,
+                int32_t out_dtype, int64_t out_stride_pass, int64_t out_stride_b, int64_t out_stride_h,
+                int64_t out_stride_l, float* lse, void* stream);
+int ra_bwd_dq_ring(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* dq,
+                   int64_t stride_pass, int64_t stride_b, int64_t stride_h, int64_t stride_l, void* stream);
+int ra_bwd_dkdv_ring(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* dk,
+                     void* dv, int64_t stride_pass, int64_t stride_b, int64_t stride_h, int64_t stride_l,
+                     void* stream);
 
 /* The elementwise entry points for the shards of n_passes passes in one launch: the fp32 arrays of
  * the passes (carries, accumulators, lse, delta) lie one after another ([n_passes, B, H, L, ...]),

@@ -219,9 +219,12 @@ void put(ra::QShardList& t, int i, const QEntry& e) {
 // launch covers them all (heaviest pass first: it is dispatched first); otherwise every pass gets
 // its own launches of at most kMaxShards steps each.  Ring is KvRing or QRing, `set_pass(ring,
 // slot, p)` fills the resident side of pass p into slot `slot`, `launch(ring)` enqueues.
+// `whole`: a whole-ring launch - passes without a live step take part too (their results are
+// still to be written), and what does not fit one launch is refused (RA_ERR_TOO_LARGE, nothing
+// launched): split into several launches a pass would need its intermediate state in memory.
 template <typename Ring, typename Table, typename Entry, typename SetPass, typename Launch>
 int run_passes(Table Ring::*table, const std::vector<Entry>& entries, const std::vector<int>& first, int n_passes,
-               SetPass set_pass, Launch launch) {
+               SetPass set_pass, Launch launch, bool whole = false) {
   std::vector<Entry> distinct;
   std::vector<int> index(entries.size());
   bool one_launch = n_passes <= ra::kMaxPasses;
@@ -242,7 +245,7 @@ int run_passes(Table Ring::*table, const std::vector<Entry>& entries, const std:
     (ring.*table).n = (int)distinct.size();
     std::vector<int> by_weight;
     for (int p = 0; p < n_passes; ++p)
-      if (first[p + 1] > first[p]) by_weight.push_back(p);
+      if (whole || first[p + 1] > first[p]) by_weight.push_back(p);
     std::stable_sort(by_weight.begin(), by_weight.end(),
                      [&](int x, int y) { return first[x + 1] - first[x] > first[y + 1] - first[y]; });
     if (by_weight.empty()) return RA_OK;
@@ -255,6 +258,9 @@ int run_passes(Table Ring::*table, const std::vector<Entry>& entries, const std:
     }
     return launch(ring);
   }
+  if (whole)
+    return fail(RA_ERR_TOO_LARGE, "a whole-ring launch takes at most %d passes that draw from at most %d distinct "
+                                  "travelling shards; use the *_passes entry points", ra::kMaxPasses, ra::kMaxShards);
   for (int p = 0; p < n_passes; ++p) {
     for (int i0 = first[p]; i0 < first[p + 1]; i0 += ra::kMaxShards) {
       const int cnt = std::min(ra::kMaxShards, first[p + 1] - i0);
@@ -283,6 +289,32 @@ bool same_bias_shape(const ra_bias& x, const ra_bias& y) {
          x.dense_stride_q == y.dense_stride_q;
 }
 
+// Where a whole-ring launch stores what it finished: pass p at `base + p * stride_pass` elements
+// (second array for dV), element size `esize`, strides in elements.
+struct RingResult {
+  void* base;
+  void* base2;
+  float* lse;
+  int dtype;  // RA_DTYPE_*
+  int64_t stride_pass, stride_b, stride_h, stride_l;
+};
+
+int check_ring_result(const char* what, const RingResult& r) {
+  if (!r.base) return fail(RA_ERR_NULL, "%s: NULL result pointer", what);
+  if (r.dtype != RA_DTYPE_BF16 && r.dtype != RA_DTYPE_F32) return fail(RA_ERR_DTYPE, "unknown out_dtype %d", r.dtype);
+  if ((r.stride_pass % 4) || (r.stride_b % 4) || (r.stride_h % 4) || (r.stride_l % 4))
+    return fail(RA_ERR_ALIGN, "%s: result strides must be multiples of 4 elements", what);
+  // the kernels store four elements at a time: 8 bytes of bf16 or 16 bytes of fp32
+  const unsigned al = r.dtype == RA_DTYPE_F32 ? 16u : 8u;
+  if (reinterpret_cast<uintptr_t>(r.base) % al || reinterpret_cast<uintptr_t>(r.base2) % al)
+    return fail(RA_ERR_ALIGN, "%s: results must be aligned to four elements (%u bytes)", what, al);
+  return RA_OK;
+}
+
+char* pass_slice(void* base, const RingResult& r, int p) {
+  return (char*)base + (int64_t)p * r.stride_pass * (r.dtype == RA_DTYPE_F32 ? 4 : 2);
+}
+
 int check_pass_counts(const int32_t* steps_per_pass, int32_t n_passes, std::vector<int>& first) {
   if (n_passes < 0) return fail(RA_ERR_SHAPE, "n_passes is negative");
   if (n_passes > 0 && !steps_per_pass) return fail(RA_ERR_NULL, "steps_per_pass is NULL");
@@ -294,7 +326,8 @@ int check_pass_counts(const int32_t* steps_per_pass, int32_t n_passes, std::vect
   return RA_OK;
 }
 
-int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream) {
+int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream,
+               const RingResult* whole = nullptr) {
   const int total = first.back();
   if (total == 0) return RA_OK;
   if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
@@ -303,13 +336,15 @@ int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, i
     for (int i = first[p]; i < first[p + 1]; ++i) {
       const ra_fwd_step_params& s = steps[i];
       const ra_fwd_step_params& h = steps[first[p]];  // head of the pass
-      int rc = ra_fwd_step_check(&s);
+      ra_fwd_step_params c = s;
+      if (whole) c.o = c.m = c.l = reinterpret_cast<float*>(uintptr_t(16));  // not used: there is no carry
+      int rc = ra_fwd_step_check(&c);
       if (rc) return rc;
       const bool shape = s.B == f.B && s.H == f.H && s.Lq == f.Lq && s.Lk == f.Lk && s.D == f.D &&
                          s.sm_scale == f.sm_scale && same_strides(s.q, f.q) && same_strides(s.k, f.k) &&
                          same_strides(s.v, f.v) && same_bias_shape(s.bias, f.bias);
-      const bool pass = !memcmp(&s.q, &h.q, sizeof(ra_tensor)) && s.o == h.o && s.m == h.m && s.l == h.l &&
-                        same_q_side(s.bias, h.bias);
+      const bool pass = !memcmp(&s.q, &h.q, sizeof(ra_tensor)) &&
+                        (whole || (s.o == h.o && s.m == h.m && s.l == h.l)) && same_q_side(s.bias, h.bias);
       if (!shape || !pass)
         return fail(RA_ERR_SHAPE, "steps[%d] differs from the first step of its pass in more than its key/value shard "
                                   "(k.ptr, v.ptr, kv_offset, kv_segment_ids, kv_prefix, dense_bias), or from "
@@ -329,6 +364,12 @@ int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, i
   a.Lk = f.Lk;
   a.scale2 = f.sm_scale * kLog2eHost;
   a.bias = to_bias(f.bias);
+  if (whole) {
+    a.bias.flags |= whole->dtype == RA_DTYPE_F32 ? ra::kFlagWholeF32 : ra::kFlagWholeBf16;
+    a.out_sb = whole->stride_b;  // in the slots of the carry pointers, which have no use here
+    a.out_sh = whole->stride_h;
+    a.out_sl = whole->stride_l;
+  }
   // live steps only: a masked step is an identity on the carry
   std::vector<KvEntry> entries;
   std::vector<int> live_first(1, 0), head(n_passes, 0);
@@ -346,6 +387,11 @@ int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, i
     r.x0[slot] = h.o;
     r.x1[slot] = h.m;
     r.x2[slot] = h.l;
+    if (whole) {
+      r.x0[slot] = reinterpret_cast<float*>(pass_slice(whole->base, *whole, p));
+      r.x1[slot] = whole->lse + (int64_t)p * f.B * f.H * f.Lq;
+      r.x2[slot] = nullptr;
+    }
     r.q_seg[slot] = h.bias.q_segment_ids;
     r.q_pre[slot] = h.bias.q_prefix;
   };
@@ -353,10 +399,11 @@ int fwd_passes(const ra_fwd_step_params* steps, const std::vector<int>& first, i
     hipError_t e = ra::launch_fwd_steps(a, r, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
     return e == hipSuccess ? RA_OK : hip_fail(e, "forward ring launch");
   };
-  return run_passes<ra::KvRing>(&ra::KvRing::kv, entries, live_first, n_passes, set_pass, launch);
+  return run_passes<ra::KvRing>(&ra::KvRing::kv, entries, live_first, n_passes, set_pass, launch, whole != nullptr);
 }
 
-int bwd_dq_passes(const ra_bwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream) {
+int bwd_dq_passes(const ra_bwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream,
+                  const RingResult* whole = nullptr) {
   const int total = first.back();
   if (total == 0) return RA_OK;
   if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
@@ -365,19 +412,27 @@ int bwd_dq_passes(const ra_bwd_step_params* steps, const std::vector<int>& first
     for (int i = first[p]; i < first[p + 1]; ++i) {
       const ra_bwd_step_params& s = steps[i];
       const ra_bwd_step_params& h = steps[first[p]];
-      int rc = ra_bwd_step_check(&s);
+      ra_bwd_step_params c = s;
+      if (whole) c.dq = c.dk = c.dv = reinterpret_cast<float*>(uintptr_t(16));  // not used: no accumulators
+      int rc = ra_bwd_step_check(&c);
       if (rc) return rc;
       const bool shape = same_dims(s, f) && same_strides(s.q, f.q) && same_strides(s.dout, f.dout) &&
                          same_strides(s.k, f.k) && same_strides(s.v, f.v) && same_bias_shape(s.bias, f.bias);
       const bool pass = !memcmp(&s.q, &h.q, sizeof(ra_tensor)) && !memcmp(&s.dout, &h.dout, sizeof(ra_tensor)) &&
-                        s.lse == h.lse && s.delta == h.delta && s.dq == h.dq && same_q_side(s.bias, h.bias);
+                        s.lse == h.lse && s.delta == h.delta && (whole || s.dq == h.dq) && same_q_side(s.bias, h.bias);
       if (!shape || !pass)
         return fail(RA_ERR_SHAPE, "steps[%d] differs from the first step of its pass in more than its key/value shard "
                                   "(k.ptr, v.ptr, dk, dv, kv_offset, kv_segment_ids, kv_prefix, dense_bias), or from "
                                   "steps[0] in shape, strides or bias terms", i);
     }
   }
-  const ra::BwdArgs a = to_bwd_args(f);
+  ra::BwdArgs a = to_bwd_args(f);
+  if (whole) {
+    a.bias.flags |= ra::kFlagWholeBf16;
+    a.out_sb = whole->stride_b;  // in the slots of the accumulator pointers, which have no use here
+    a.out_sh = whole->stride_h;
+    a.out_sl = whole->stride_l;
+  }
   std::vector<KvEntry> entries;
   std::vector<int> live_first(1, 0);
   for (int p = 0; p < n_passes; ++p) {
@@ -391,7 +446,7 @@ int bwd_dq_passes(const ra_bwd_step_params* steps, const std::vector<int>& first
     r.q_off[slot] = (int)h.bias.q_offset;
     r.q[slot] = (const ra::bf16_t*)h.q.ptr;
     r.dout[slot] = (const ra::bf16_t*)h.dout.ptr;
-    r.x0[slot] = h.dq;
+    r.x0[slot] = whole ? reinterpret_cast<float*>(pass_slice(whole->base, *whole, p)) : h.dq;
     r.x1[slot] = const_cast<float*>(h.lse);
     r.x2[slot] = const_cast<float*>(h.delta);
     r.q_seg[slot] = h.bias.q_segment_ids;
@@ -401,10 +456,11 @@ int bwd_dq_passes(const ra_bwd_step_params* steps, const std::vector<int>& first
     hipError_t e = ra::launch_bwd_dq_steps(a, r, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
     return e == hipSuccess ? RA_OK : hip_fail(e, "dQ ring launch");
   };
-  return run_passes<ra::KvRing>(&ra::KvRing::kv, entries, live_first, n_passes, set_pass, launch);
+  return run_passes<ra::KvRing>(&ra::KvRing::kv, entries, live_first, n_passes, set_pass, launch, whole != nullptr);
 }
 
-int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream) {
+int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& first, int n_passes, void* stream,
+                    const RingResult* whole = nullptr) {
   const int total = first.back();
   if (total == 0) return RA_OK;
   if (!steps) return fail(RA_ERR_NULL, "steps is NULL");
@@ -413,19 +469,27 @@ int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& fir
     for (int i = first[p]; i < first[p + 1]; ++i) {
       const ra_bwd_step_params& s = steps[i];
       const ra_bwd_step_params& h = steps[first[p]];
-      int rc = ra_bwd_step_check(&s);
+      ra_bwd_step_params c = s;
+      if (whole) c.dq = c.dk = c.dv = reinterpret_cast<float*>(uintptr_t(16));  // not used: no accumulators
+      int rc = ra_bwd_step_check(&c);
       if (rc) return rc;
       const bool shape = same_dims(s, f) && same_strides(s.q, f.q) && same_strides(s.dout, f.dout) &&
                          same_strides(s.k, f.k) && same_strides(s.v, f.v) && same_bias_shape(s.bias, f.bias);
       const bool pass = !memcmp(&s.k, &h.k, sizeof(ra_tensor)) && !memcmp(&s.v, &h.v, sizeof(ra_tensor)) &&
-                        s.dk == h.dk && s.dv == h.dv && same_kv_side(s.bias, h.bias);
+                        (whole || (s.dk == h.dk && s.dv == h.dv)) && same_kv_side(s.bias, h.bias);
       if (!shape || !pass)
         return fail(RA_ERR_SHAPE, "steps[%d] differs from the first step of its pass in more than its query shard (q.ptr, "
                                   "dout.ptr, lse, delta, dq, q_offset, q_segment_ids, q_prefix, dense_bias), or from "
                                   "steps[0] in shape, strides or bias terms", i);
     }
   }
-  const ra::BwdArgs a = to_bwd_args(f);
+  ra::BwdArgs a = to_bwd_args(f);
+  if (whole) {
+    a.bias.flags |= ra::kFlagWholeBf16;
+    a.out_sb = whole->stride_b;  // in the slots of the accumulator pointers, which have no use here
+    a.out_sh = whole->stride_h;
+    a.out_sl = whole->stride_l;
+  }
   std::vector<QEntry> entries;
   std::vector<int> live_first(1, 0);
   for (int p = 0; p < n_passes; ++p) {
@@ -439,8 +503,8 @@ int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& fir
     r.kv_off[slot] = (int)h.bias.kv_offset;
     r.k[slot] = (const ra::bf16_t*)h.k.ptr;
     r.v[slot] = (const ra::bf16_t*)h.v.ptr;
-    r.dk[slot] = h.dk;
-    r.dv[slot] = h.dv;
+    r.dk[slot] = whole ? reinterpret_cast<float*>(pass_slice(whole->base, *whole, p)) : h.dk;
+    r.dv[slot] = whole ? reinterpret_cast<float*>(pass_slice(whole->base2, *whole, p)) : h.dv;
     r.kv_seg[slot] = h.bias.kv_segment_ids;
     r.kv_pre[slot] = h.bias.kv_prefix;
   };
@@ -448,14 +512,14 @@ int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& fir
     hipError_t e = ra::launch_bwd_dkdv_steps(a, r, f.D, kernel_mode(f.bias.flags), (hipStream_t)stream);
     return e == hipSuccess ? RA_OK : hip_fail(e, "dK/dV ring launch");
   };
-  return run_passes<ra::QRing>(&ra::QRing::q, entries, live_first, n_passes, set_pass, launch);
+  return run_passes<ra::QRing>(&ra::QRing::q, entries, live_first, n_passes, set_pass, launch, whole != nullptr);
 }
 
 }  // namespace
 
 extern "C" {
 
-int ra_version(void) { return 1004; }
+int ra_version(void) { return 1005; }
 
 const char* ra_last_error(void) { return g_err; }
 
@@ -635,6 +699,47 @@ int ra_bwd_dkdv_passes(const ra_bwd_step_params* steps, const int32_t* steps_per
   std::vector<int> first;
   int rc = check_pass_counts(steps_per_pass, n_passes, first);
   return rc ? rc : bwd_dkdv_passes(steps, first, n_passes, stream);
+}
+
+// every pass of a whole-ring launch needs a head block to take its resident side from
+static int check_whole(const std::vector<int>& first, int n_passes) {
+  for (int p = 0; p < n_passes; ++p)
+    if (first[p + 1] == first[p]) return fail(RA_ERR_SHAPE, "pass %d has no block", p);
+  return RA_OK;
+}
+
+int ra_fwd_ring(const ra_fwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* out,
+                int32_t out_dtype, int64_t out_stride_pass, int64_t out_stride_b, int64_t out_stride_h,
+                int64_t out_stride_l, float* lse, void* stream) {
+  std::vector<int> first;
+  int rc = check_pass_counts(steps_per_pass, n_passes, first);
+  if (rc || (rc = check_whole(first, n_passes))) return rc;
+  if (!lse) return fail(RA_ERR_NULL, "ra_fwd_ring: lse is NULL");
+  const RingResult r{out, nullptr, lse, out_dtype, out_stride_pass, out_stride_b, out_stride_h, out_stride_l};
+  if ((rc = check_ring_result("ra_fwd_ring", r))) return rc;
+  return fwd_passes(steps, first, n_passes, stream, &r);
+}
+
+int ra_bwd_dq_ring(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* dq,
+                   int64_t stride_pass, int64_t stride_b, int64_t stride_h, int64_t stride_l, void* stream) {
+  std::vector<int> first;
+  int rc = check_pass_counts(steps_per_pass, n_passes, first);
+  if (rc || (rc = check_whole(first, n_passes))) return rc;
+  const RingResult r{dq, nullptr, nullptr, RA_DTYPE_BF16, stride_pass, stride_b, stride_h, stride_l};
+  if ((rc = check_ring_result("ra_bwd_dq_ring", r))) return rc;
+  return bwd_dq_passes(steps, first, n_passes, stream, &r);
+}
+
+int ra_bwd_dkdv_ring(const ra_bwd_step_params* steps, const int32_t* steps_per_pass, int32_t n_passes, void* dk,
+                     void* dv, int64_t stride_pass, int64_t stride_b, int64_t stride_h, int64_t stride_l,
+                     void* stream) {
+  std::vector<int> first;
+  int rc = check_pass_counts(steps_per_pass, n_passes, first);
+  if (rc || (rc = check_whole(first, n_passes))) return rc;
+  if (!dv) return fail(RA_ERR_NULL, "ra_bwd_dkdv_ring: dv is NULL");
+  const RingResult r{dk, dv, nullptr, RA_DTYPE_BF16, stride_pass, stride_b, stride_h, stride_l};
+  if ((rc = check_ring_result("ra_bwd_dkdv_ring", r))) return rc;
+  return bwd_dkdv_passes(steps, first, n_passes, stream, &r);
 }
 
 int ra_bwd_finalize_passes(const float* acc, void* out, int64_t out_stride_pass, int64_t out_stride_b,

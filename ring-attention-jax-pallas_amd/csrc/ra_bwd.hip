@@ -926,7 +926,28 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     compute_dkdv(pf, dsf, s_q[0] + last * TILE_BYTES, s_do[0] + last * TILE_BYTES);
   }
   }  // query shards
-  if (tiles_listed == 0) return;  // nothing to add
+  const bool whole_ring = MULTI && (flags & kFlagWhole);
+  if (!whole_ring && tiles_listed == 0) return;  // nothing to add
+  if constexpr (MULTI) {
+    if (whole_ring) {
+      // the gradients of this key slab are complete: bf16, in the caller's layout
+      const long long at = b * a.out_sb + h * a.out_sh + (long long)(kw + 4 * g) * a.out_sl + l32;
+      bf16_t* const dkp = (bf16_t*)ring.dk[blockIdx.y] + at;
+      bf16_t* const dvp = (bf16_t*)ring.dv[blockIdx.y] + at;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kr = 8 * (r / 4) + (r % 4);
+        if (kw + 4 * g + kr < a.Lk) {
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            dkp[kr * a.out_sl + 32 * db] = (bf16_t)(dk[db][r] * a.sm_scale);
+            dvp[kr * a.out_sl + 32 * db] = (bf16_t)dv[db][r];
+          }
+        }
+      }
+      return;
+    }
+  }
   // ---- accumulate into the fp32 gradients owned by this key slab ------------------------------
   // All loads of an array are issued before the first value is needed: a load - add - store chain
   // per element would cost one memory round trip each, a hundred in a row with nothing to hide them.
@@ -1840,7 +1861,26 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     compute_dq(dsf, s_k[0] + ((n - 1) % NBUF) * TILE_BYTES);
   }
   }  // key/value shards
-  if (tiles_listed == 0) return;  // nothing to add
+  const bool whole_ring = MULTI && (flags & kFlagWhole);
+  if (!whole_ring && tiles_listed == 0) return;  // nothing to add
+  if constexpr (MULTI) {
+    if (whole_ring) {
+      // dQ of these rows is complete: bf16, in the caller's layout
+      if (q_valid) {
+        bf16_t* dq = (bf16_t*)ring.x0[blockIdx.y] + b * a.out_sb + h * a.out_sh + (long long)qi * a.out_sl + 4 * g;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int bb = 0; bb < 4; ++bb) {
+            bf16x4 t;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) t[c] = (bf16_t)(acc[db][4 * bb + c] * a.sm_scale);
+            *(bf16x4*)(dq + 32 * db + 8 * bb) = t;
+          }
+      }
+      return;
+    }
+  }
   if (q_valid) {
     float* dq_res = a.dq;
     if constexpr (MULTI) dq_res = ring.x0[blockIdx.y];

@@ -23,9 +23,12 @@ constexpr int kPlainMinTiles = 16;  // shortest stretch of plain tiles that take
 // walks the key/value shards that `ring` lists for the pass one after another (the arguments of
 // consecutive ring steps of that query shard); the step's contribution stays in registers between
 // them and meets the carry of the pass once, at the end.
-template <int D, int MODE, bool MULTI>
+// WHOLE: a whole-ring launch (see kFlagWhole) - its own instantiation: the variants that merge a
+// carry keep the register allocation they have without the extra exit path.
+template <int D, int MODE, bool MULTI, bool WHOLE = false>
 __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const FwdArgs a, const std::conditional_t<MULTI, KvRing, NoShardList> ring) {
+  static_assert(MULTI || !WHOLE, "a whole-ring launch walks the shards of its passes itself");
   constexpr bool GENERAL = MODE != 0;  // bias terms beyond causal / window
   constexpr bool DENSE = MODE == 2;    // ... including a materialised bias block
   constexpr int KS = D / 16;  // k-steps of the QK^T contraction
@@ -106,7 +109,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // l_run / lr_run makes it a properly normalised average of V times the exact row sum, so
   // the rounding of P cancels in o / l instead of showing up as an error of order 2^-9 |v|
   // on rows that see only a few keys.
-  float m_run = pass_m()[row] * kLog2e;  // exponent reference (log2 domain), moves lazily
+  // whole-ring launch: no carry comes in, the finished output goes out
+  float m_run = WHOLE ? RA_NEG_INF : pass_m()[row] * kLog2e;  // exponent reference (log2 domain), moves lazily
   float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
   // In a long stretch of completely unmasked tiles (at least kPlainMinTiles of them) a tile adds
   // only its ROUNDED probabilities, to this third sum, which counts for both l and lr: the
@@ -1049,7 +1053,45 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // A wave that gathered no probability mass (no tile listed for its workgroup, or every score
   // masked) has nothing to merge: with l_step = 0 and an unchanged maximum the merge below is the
   // identity, so the carry's 32 rows stay where they are, unread.
-  if (__all(l_run == 0.f && lr_run == 0.f && lp_run == 0.f)) return;
+  if (!WHOLE && __all(l_run == 0.f && lr_run == 0.f && lp_run == 0.f)) return;
+  if constexpr (WHOLE) {
+    {
+      // out = o_step / (sum of the rounded weights): the normalised average of V;
+      // lse = ln 2 (m_run + log2 l_step) with the exact sum.  A row that saw no key: 0 / 0 and -inf.
+      const int qi_out = q0 + wave * 32 + l32;
+      row = ((long long)b * a.H + h) * a.Lq + min(qi_out, a.Lq - 1);
+      const float l_step = half_sum(l_run + lp_run), lr_step = half_sum(lr_run + lp_run);
+      const float inv = 1.0f / lr_step;
+      if (q_valid) {
+        const long long at = b * a.out_sb + h * a.out_sh + (long long)qi_out * a.out_sl + 4 * g;
+        if (flags & kFlagWholeBf16) {
+          bf16_t* op = (bf16_t*)ring.x0[blockIdx.y] + at;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) {
+              bf16x4 t;
+#pragma unroll
+              for (int c = 0; c < 4; ++c) t[c] = (bf16_t)(oacc[db][4 * bb + c] * inv);
+              *(bf16x4*)(op + 32 * db + 8 * bb) = t;
+            }
+        } else {
+          float* op = ring.x0[blockIdx.y] + at;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) {
+              f32x4 t;
+#pragma unroll
+              for (int c = 0; c < 4; ++c) t[c] = oacc[db][4 * bb + c] * inv;
+              *(f32x4*)(op + 32 * db + 8 * bb) = t;
+            }
+        }
+        if (g == 0) ring.x1[blockIdx.y][row] = (l_step > 0.f) ? (m_run + __log2f(l_step)) * kLn2 : RA_NEG_INF;
+      }
+      return;
+    }
+  }
   // ---- merge this step into the carry ---------------------------------------------------------
   // o = o_in 2^(m_in - m_out) + o_step 2^(m_run - m_out) l_step / lr_step,  l likewise with the
   // exact sum, m_out = exact maximum over carry and step.
@@ -1133,28 +1175,29 @@ __global__ void fwd_finalize_kernel(const float* o, const float* m, const float*
 namespace ra {
 
 // mode: 0 = causal / window terms only, 1 = any of the per-tile terms, 2 = a dense bias block too
-template <bool MULTI, typename Shards>
+template <bool MULTI, bool WHOLE, typename Shards>
 static hipError_t launch_fwd(const FwdArgs& a, const Shards& sl, int n_pass, int D, int mode, hipStream_t stream) {
   const int nqt = (a.Lq + kFwdRows - 1) / kFwdRows;
   dim3 grid((unsigned)(a.B * a.H * nqt), (unsigned)n_pass), block(kFwdThreads);
   if (D == 128) {
-    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<128, 2, MULTI>), grid, block, 0, stream, a, sl);
-    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<128, 1, MULTI>), grid, block, 0, stream, a, sl);
-    else hipLaunchKernelGGL((fwd_step_kernel<128, 0, MULTI>), grid, block, 0, stream, a, sl);
+    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<128, 2, MULTI, WHOLE>), grid, block, 0, stream, a, sl);
+    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<128, 1, MULTI, WHOLE>), grid, block, 0, stream, a, sl);
+    else hipLaunchKernelGGL((fwd_step_kernel<128, 0, MULTI, WHOLE>), grid, block, 0, stream, a, sl);
   } else {
-    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<64, 2, MULTI>), grid, block, 0, stream, a, sl);
-    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<64, 1, MULTI>), grid, block, 0, stream, a, sl);
-    else hipLaunchKernelGGL((fwd_step_kernel<64, 0, MULTI>), grid, block, 0, stream, a, sl);
+    if (mode == 2) hipLaunchKernelGGL((fwd_step_kernel<64, 2, MULTI, WHOLE>), grid, block, 0, stream, a, sl);
+    else if (mode == 1) hipLaunchKernelGGL((fwd_step_kernel<64, 1, MULTI, WHOLE>), grid, block, 0, stream, a, sl);
+    else hipLaunchKernelGGL((fwd_step_kernel<64, 0, MULTI, WHOLE>), grid, block, 0, stream, a, sl);
   }
   return hipGetLastError();
 }
 
 hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream) {
-  return launch_fwd<false>(a, NoShardList{}, 1, D, mode, stream);
+  return launch_fwd<false, false>(a, NoShardList{}, 1, D, mode, stream);
 }
 
 hipError_t launch_fwd_steps(const FwdArgs& a, const KvRing& ring, int D, int mode, hipStream_t stream) {
-  return launch_fwd<true>(a, ring, ring.n_pass, D, mode, stream);
+  if (a.bias.flags & kFlagWhole) return launch_fwd<true, true>(a, ring, ring.n_pass, D, mode, stream);
+  return launch_fwd<true, false>(a, ring, ring.n_pass, D, mode, stream);
 }
 
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream) {

@@ -5,11 +5,23 @@
 
 namespace ra {
 
+// Whole-ring launches (every step of a pass in one launch, several-shard kernels only) are marked
+// by one of these bits in BiasArgs::flags, next to the RA_BIAS_* bits.  Forward: the carry starts
+// empty and never touches memory; the pass's x0 / x1 table entries are its slice of the attention
+// output (bf16 or fp32) and its logsumexp rows.  Backward: the gradient of the resident shard is
+// complete when its workgroup ends and is stored as bf16 where the pass's accumulator entries
+// point, instead of being added to fp32 accumulators.  The strides of those results (in
+// elements) travel in the argument slots of the pointers that such a launch does not use, so
+// that the argument block does not grow: the kernels' scalar registers are all taken.
+constexpr int kFlagWholeBf16 = 1 << 24;
+constexpr int kFlagWholeF32 = 1 << 25;
+constexpr int kFlagWhole = kFlagWholeBf16 | kFlagWholeF32;
+
 struct FwdArgs {
   TensorArg q, k, v;
-  float* o;
-  float* m;
-  float* l;
+  union { float* o; long long out_sb; };
+  union { float* m; long long out_sh; };
+  union { float* l; long long out_sl; };
   int B, H, Lq, Lk;
   float scale2;  // sm_scale * log2(e)
   BiasArgs bias;
@@ -19,9 +31,9 @@ struct BwdArgs {
   TensorArg q, k, v, dout;
   const float* lse;
   const float* delta;
-  float* dq;
-  float* dk;
-  float* dv;
+  union { float* dq; long long out_sb; };
+  union { float* dk; long long out_sh; };
+  union { float* dv; long long out_sl; };
   int B, H, Lq, Lk;
   float scale2;    // sm_scale * log2(e) = scale_p2 * scale_res
   float scale_p2;  // the power of two below scale2: folded into a bf16 operand without rounding

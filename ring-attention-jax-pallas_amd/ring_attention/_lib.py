@@ -14,6 +14,7 @@ RA_BIAS_PREFIX = 8
 RA_BIAS_ALIBI = 16
 RA_BIAS_DENSE = 32
 RA_DTYPE_BF16 = 0
+RA_ERR_TOO_LARGE = -8  # a whole-ring launch cannot hold the passes: use the split entry points
 RA_DTYPE_F32 = 1
 
 
@@ -77,6 +78,12 @@ EXPORTS = {
     "ra_fwd_passes": (C.c_int, [C.POINTER(RaFwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p]),
     "ra_bwd_dq_passes": (C.c_int, [C.POINTER(RaBwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p]),
     "ra_bwd_dkdv_passes": (C.c_int, [C.POINTER(RaBwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p]),
+    "ra_fwd_ring": (C.c_int, [C.POINTER(RaFwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p, C.c_int32,
+                              C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
+    "ra_bwd_dq_ring": (C.c_int, [C.POINTER(RaBwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p, C.c_int64,
+                                 C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
+    "ra_bwd_dkdv_ring": (C.c_int, [C.POINTER(RaBwdStepParams), C.POINTER(C.c_int32), C.c_int32, C.c_void_p,
+                                   C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_void_p]),
     "ra_fwd_finalize_passes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int64,
                                          C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_int32, C.c_int32,
                                          C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),

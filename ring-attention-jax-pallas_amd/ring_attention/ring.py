@@ -128,10 +128,11 @@ def _fwd_params(q, k, v, bias, o, m, l, sm_scale) -> _lib.RaFwdStepParams:
     p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
     p.sm_scale = float(sm_scale)
     p.q, p.k, p.v = _view_bhld(q), _view_bhld(k), _view_bhld(v)
-    for t_ in (o, m, l):
-        if t_.dtype != torch.float32 or not t_.is_contiguous():
-            raise ValueError("o, m, l carries must be contiguous float32 tensors")
-    p.o, p.m, p.l = o.data_ptr(), m.data_ptr(), l.data_ptr()
+    if o is not None:  # None: the caller fills the carry pointers in later, or has no carry
+        for t_ in (o, m, l):
+            if t_.dtype != torch.float32 or not t_.is_contiguous():
+                raise ValueError("o, m, l carries must be contiguous float32 tensors")
+        p.o, p.m, p.l = o.data_ptr(), m.data_ptr(), l.data_ptr()
     p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
     return p
 
@@ -205,7 +206,8 @@ def _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale) -> _lib.RaB
     p.sm_scale = float(sm_scale)
     p.q, p.k, p.v, p.dout = _view_bhld(q), _view_bhld(k), _view_bhld(v), _view_bhld(do)
     p.lse, p.delta = lse.data_ptr(), delta.data_ptr()
-    p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+    if dq is not None:  # None: the caller fills the accumulator pointers in later, or has none
+        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
     p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
     return p
 
@@ -480,19 +482,19 @@ def _pass_steps(plan: "_RingPlan", cache_key, key, build):
     return hit[1:]
 
 
-def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO_TIMER):
+def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO_TIMER, whole=True):
     """``_ring_forward`` with ALL ring passes in one launch: grid dimension y is the query shard,
-    and the kernel visits that shard's key/value shards in ring order itself.  Three launches per
-    forward: carry reset, the ring, finalisation."""
+    and the kernel visits that shard's key/value shards in ring order itself.  ``whole``: the one
+    launch is everything (ra_fwd_ring: the carry of ring.py:104-132 stays in registers, output and
+    logsumexp come out finished); a ring too large for that, or ``whole=False``, takes three
+    launches: carry reset, the ring (ra_fwd_passes), finalisation."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     lib = _lib.load()
     out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
     lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    o = torch.empty((n, B, H, Lq, D), dtype=torch.float32, device=dev)
-    m = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    l = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
-    _lib.check("ra_fwd_init", lib.ra_fwd_init(o.data_ptr(), m.data_ptr(), l.data_ptr(), n * B, H, Lq, D, _stream()))
+    dt = {torch.bfloat16: _lib.RA_DTYPE_BF16, torch.float32: _lib.RA_DTYPE_F32}[out.dtype]
+    ov = out.permute(0, 2, 1, 3)  # [b, h, S, d] view; shard r starts r * Lq rows further
 
     def build():
         steps = (_lib.RaFwdStepParams * (n * n))()
@@ -503,13 +505,24 @@ def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO
                 bias = plan.block_bias(r, src)
                 keep.append(bias)
                 steps[r * n + t] = _fwd_params(_shard_bhld(q, r, Lq), _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk),
-                                               bias, o[r], m[r], l[r], sm_scale)
+                                               bias, None, None, None, sm_scale)  # carry pointers: set per call
         return steps, (C.c_int32 * n)(*([n] * n)), keep
 
     key = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(), k.stride(), v.stride(), sm_scale)
     steps, counts, _keep = _pass_steps(plan, "fwd", key, build)
     if plan.callable is not None:
         steps, counts, _keep = build()  # a callable's dense blocks are fresh tensors every time
+    if whole:
+        with timer.span("fwd_ring", -1, -1):
+            rc = lib.ra_fwd_ring(steps, counts, n, out.data_ptr(), dt, Lq * ov.stride(2), ov.stride(0), ov.stride(1),
+                                 ov.stride(2), lse.data_ptr(), _stream())
+        if rc != _lib.RA_ERR_TOO_LARGE:
+            _lib.check("ra_fwd_ring", rc)
+            return out, lse
+    o = torch.empty((n, B, H, Lq, D), dtype=torch.float32, device=dev)
+    m = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    l = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    _lib.check("ra_fwd_init", lib.ra_fwd_init(o.data_ptr(), m.data_ptr(), l.data_ptr(), n * B, H, Lq, D, _stream()))
     so, sm = o[0].numel() * 4, m[0].numel() * 4
     for r in range(n):
         for t in range(n):
@@ -517,18 +530,19 @@ def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO
             st.o, st.m, st.l = o.data_ptr() + r * so, m.data_ptr() + r * sm, l.data_ptr() + r * sm
     with timer.span("fwd_ring", -1, -1):
         _lib.check("ra_fwd_passes", lib.ra_fwd_passes(steps, counts, n, _stream()))
-    dt = {torch.bfloat16: _lib.RA_DTYPE_BF16, torch.float32: _lib.RA_DTYPE_F32}[out.dtype]
-    ov = out.permute(0, 2, 1, 3)  # [b, h, S, d] view; shard r starts r * Lq rows further
     _lib.check("ra_fwd_finalize_passes", lib.ra_fwd_finalize_passes(
         o.data_ptr(), m.data_ptr(), l.data_ptr(), out.data_ptr(), dt, Lq * ov.stride(2), ov.stride(0), ov.stride(1),
         ov.stride(2), lse.data_ptr(), n, B, H, Lq, D, _stream()))
     return out, lse
 
 
-def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER):
+def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer=_NO_TIMER, whole=True):
     """``_ring_backward`` with all passes of a kind in one launch: one for dK / dV (grid dimension y
     is the key/value shard, the kernel visits the query shards in the order they arrive,
-    ring.py:195), one for dQ (y is the query shard), around one delta launch and three casts."""
+    ring.py:195), one for dQ (y is the query shard), behind one delta launch.  ``whole``: the two
+    launches store the finished bf16 gradients themselves (ra_bwd_dkdv_ring, ra_bwd_dq_ring); a
+    ring too large for that, or ``whole=False``, adds into zeroed fp32 accumulators
+    (ra_bwd_*_passes) that three more launches cast."""
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     lib = _lib.load()
@@ -539,8 +553,6 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
     _lib.check("ra_bwd_delta_passes", lib.ra_bwd_delta_passes(
         out.data_ptr(), dt, Lq * ov.stride(2), ov.stride(0), ov.stride(1), ov.stride(2), C.byref(do_t),
         Lq * dov.stride(2), delta.data_ptr(), n, B, H, Lq, D, _stream()))
-    dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
-    dkv_acc = torch.zeros((2, n, B, H, Lk, D), dtype=torch.float32, device=dev)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
 
     def build():
@@ -555,8 +567,8 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
                     bias = plan.block_bias(qs, ks)
                     keep.append(bias)
                     arr[r * n + t] = _bwd_params(_shard_bhld(q, qs, Lq), _shard_bhld(k, ks, Lk), _shard_bhld(v, ks, Lk),
-                                                 _shard_bhld(do, qs, Lq), lse[qs], delta[qs], dq_acc[qs],
-                                                 dkv_acc[0, ks], dkv_acc[1, ks], bias, sm_scale)
+                                                 _shard_bhld(do, qs, Lq), lse[qs], delta[qs], None, None, None,
+                                                 bias, sm_scale)  # accumulator pointers: set per call
         pairs = [((r - t) % n, r) for r in range(n) for t in range(n)], [(r, (r + t) % n) for r in range(n) for t in range(n)]
         return by_kv, by_q, pairs, (C.c_int32 * n)(*([n] * n)), keep
 
@@ -564,7 +576,7 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
     by_kv, by_q, pairs, counts, _keep = _pass_steps(plan, "bwd", key, build)
     if plan.callable is not None:
         by_kv, by_q, pairs, counts, _keep = build()
-    s_row, s_acc, s_kv = lse[0].numel() * 4, dq_acc[0].numel() * 4, dkv_acc[0, 0].numel() * 4
+    s_row = lse[0].numel() * 4
     do_shard = Lq * do.stride(1) * do.element_size()
     for arr, pr in zip((by_kv, by_q), pairs):
         for i, (qs, ks) in enumerate(pr):
@@ -572,6 +584,24 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
             st.dout.ptr = do.data_ptr() + qs * do_shard
             st.dout.stride_b, st.dout.stride_h, st.dout.stride_l = do.stride(0), do.stride(2), do.stride(1)
             st.lse, st.delta = lse.data_ptr() + qs * s_row, delta.data_ptr() + qs * s_row
+    if whole:
+        gq, gk, gv = (g.permute(0, 2, 1, 3) for g in (dq, dk, dv))
+        assert gk.stride() == gv.stride()
+        with timer.span("bwd_dkdv_ring", -1, -1):
+            rc = lib.ra_bwd_dkdv_ring(by_kv, counts, n, dk.data_ptr(), dv.data_ptr(), Lk * gk.stride(2), gk.stride(0),
+                                      gk.stride(1), gk.stride(2), _stream())
+        if rc != _lib.RA_ERR_TOO_LARGE:
+            _lib.check("ra_bwd_dkdv_ring", rc)
+            with timer.span("bwd_dq_ring", -1, -1):
+                _lib.check("ra_bwd_dq_ring", lib.ra_bwd_dq_ring(by_q, counts, n, dq.data_ptr(), Lq * gq.stride(2),
+                                                                gq.stride(0), gq.stride(1), gq.stride(2), _stream()))
+            return dq, dk, dv
+    dq_acc = torch.zeros((n, B, H, Lq, D), dtype=torch.float32, device=dev)
+    dkv_acc = torch.zeros((2, n, B, H, Lk, D), dtype=torch.float32, device=dev)
+    s_acc, s_kv = dq_acc[0].numel() * 4, dkv_acc[0, 0].numel() * 4
+    for arr, pr in zip((by_kv, by_q), pairs):
+        for i, (qs, ks) in enumerate(pr):
+            st = arr[i]
             st.dq = dq_acc.data_ptr() + qs * s_acc
             st.dk = dkv_acc.data_ptr() + ks * s_kv
             st.dv = dkv_acc.data_ptr() + (n + ks) * s_kv

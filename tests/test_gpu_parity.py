@@ -523,8 +523,8 @@ def test_pass_entry_points_equal_launches_per_pass(device):
     plan = rr._RingPlan(q, k, n, ra.causal_bias() + ra.segment_bias(), {"q_segment_ids": seg}, {"kv_segment_ids": seg})
     sc = 1 / math.sqrt(D)
     sh = lambda x, s_: rr._shard_bhld(x, s_, L)
-    out, lse = rr._ring_forward_fused(q, k, v, plan, sc, torch.float32)
-    dq, dk, dv = rr._ring_backward_fused(q, k, v, out, lse, do, plan, sc)
+    out, lse = rr._ring_forward_fused(q, k, v, plan, sc, torch.float32, whole=False)
+    dq, dk, dv = rr._ring_backward_fused(q, k, v, out, lse, do, plan, sc, whole=False)
     # the same passes, one launch each
     out1 = torch.empty_like(out)
     lse1 = torch.empty_like(lse)
@@ -550,9 +550,40 @@ def test_pass_entry_points_equal_launches_per_pass(device):
     torch.cuda.synchronize()
     assert torch.equal(dq, dq1) and torch.equal(dk, dk1) and torch.equal(dv, dv1)
     # a second call reuses the cached parameter blocks of the plan with fresh buffers
-    out2, lse2 = rr._ring_forward_fused(q, k, v, plan, sc, torch.float32)
-    g2 = rr._ring_backward_fused(q, k, v, out2, lse2, do, plan, sc)
+    out2, lse2 = rr._ring_forward_fused(q, k, v, plan, sc, torch.float32, whole=False)
+    g2 = rr._ring_backward_fused(q, k, v, out2, lse2, do, plan, sc, whole=False)
     assert torch.equal(out2, out) and all(torch.equal(a, b_) for a, b_ in zip(g2, (dq, dk, dv)))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_whole_ring_entry_points_agree_with_the_split_ones(device, out_dtype):
+    """ra_fwd_ring / ra_bwd_dq_ring / ra_bwd_dkdv_ring (nothing between the launches goes through
+    memory) against init + ra_*_passes + finalize on the same inputs: the same sums, the final
+    division and casts folded differently, so they agree to rounding - fp32 outputs to 1e-5 relative,
+    bf16 results to one unit in the last place.  Cross attention with a window leaves query rows
+    without any key (NaN output, -inf logsumexp, zero gradient) and a pass without a live step."""
+    B, H, D, n, Lq, Lk = 2, 2, 128, 4, 320, 192
+    q, k, v, do = R.make_inputs(23, B, n * Lq, n * Lk, H, D)
+    q, k, v, do = (_dev(x, device, torch.bfloat16) for x in (q, k, v, do))
+    sc = 1 / math.sqrt(D)
+    for fn in (None, ra.causal_bias(), ra.sliding_window_bias(100)):
+        plan = rr._RingPlan(q, k, n, fn, None, None)
+        outs = [rr._ring_forward_fused(q, k, v, plan, sc, out_dtype, whole=w) for w in (True, False)]
+        (o1, l1), (o0, l0) = outs
+        assert torch.equal(torch.isnan(o1), torch.isnan(o0)) and torch.equal(torch.isinf(l1), torch.isinf(l0))
+        fin = ~torch.isnan(o0)
+        tol = 1e-5 if out_dtype == torch.float32 else 2.0 ** -7
+        assert ((o1.float() - o0.float()).abs()[fin] <= tol * o0.float().abs()[fin] + 1e-6).all()
+        lf = ~torch.isinf(l0)
+        assert ((l1 - l0).abs()[lf] <= 1e-5).all()
+        out_b = torch.nan_to_num(o0).to(torch.bfloat16)
+        lse_b = l0
+        g1 = rr._ring_backward_fused(q, k, v, out_b, lse_b, do, plan, sc, whole=True)
+        g0 = rr._ring_backward_fused(q, k, v, out_b, lse_b, do, plan, sc, whole=False)
+        torch.cuda.synchronize()
+        for a, b_ in zip(g1, g0):
+            assert torch.isfinite(a.float()).all()
+            assert ((a.float() - b_.float()).abs() <= 2.0 ** -7 * b_.float().abs() + 1e-6).all()
 
 
 def test_fused_ring_pass_with_a_callable_bias_fn(device):
