@@ -181,6 +181,31 @@ def test_long_documents(device, causal, ring):
            std=0.7)
 
 
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+@pytest.mark.parametrize("causal,D", [(False, 128), (True, 128), (False, 64)])
+def test_documents_and_alibi_inside_the_straight_line_loops(device, impl, causal, D):
+    """Documents + ALiBi (C4's bias) on documents long enough for straight-line stretches in all
+    three kernels: a document shorter than a workgroup's rows (100 tokens), a workgroup that
+    straddles a boundary off the tile grid (two runs of one-id tiles: 1500 lies inside rows
+    1280-1535), a document that crosses the shard boundary, ALiBi stretches on both sides of
+    the diagonal (not causal) or one (causal), one slope per head."""
+    S, H = 4096, 4
+    seg = np.zeros((1, S), np.int32)
+    seg[0, 100:1500] = 1
+    seg[0, 1500:] = 2
+    sl = R.alibi_slopes(H)
+    fn = ra.segment_bias() + ra.alibi_bias(sl)
+    if causal:
+        fn = fn + ra.causal_bias()
+    _check(device, f"documents+alibi causal={causal} D={D}", 1, S, S, H, D, 2, fn,
+           R.make_bias_fn(causal=causal, use_segments=True, alibi=sl), {"q_segment_ids": seg},
+           {"kv_segment_ids": seg}, impl=impl)
+    # ALiBi alone: every tile off the diagonal band is inside a stretch
+    fn = ra.alibi_bias(sl) + ra.causal_bias() if causal else ra.alibi_bias(sl)
+    _check(device, f"alibi causal={causal} D={D}", 1, S, S, H, D, 2, fn, R.make_bias_fn(causal=causal, alibi=sl),
+           impl=impl, seed=3)
+
+
 def test_fully_masked_rows_do_not_poison_key_gradients(device):
     # queries whose segment id matches no key: o = NaN, lse = -inf like the reference
     # (ring.py:134-135); such rows must contribute nothing to dk / dv.  The expected gradients
