@@ -1015,7 +1015,8 @@ def test_config3_full_size(device):
                      _causal_row_np(S), heads={0, 13, H - 1})
 
 
-def test_config4_full_size(device):
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_config4_full_size(device, impl):
     # B=1 H=16 D=128 S=32768 in 4 shards: geometric segments (mean 2048) + ALiBi 2^(-8h/H)
     B, H, D, S, n = 1, 16, 128, 32768, 4
     seg = R.geometric_segment_ids(0, B, S, 2048)
@@ -1031,11 +1032,12 @@ def test_config4_full_size(device):
 
     brow = lambda b, h, i: np.where(seg[b] == seg[b, i], 0.0, -np.inf) - slopes[h] * np.abs(i - pos)
     _full_size_check(device, "C4", B, H, D, S, n, ra.segment_bias() + ra.alibi_bias(slopes), 1.0, rows_t, brow,
-                     {"q_segment_ids": tseg}, {"kv_segment_ids": tseg}, heads={0, 7, H - 1})
+                     {"q_segment_ids": tseg}, {"kv_segment_ids": tseg}, impl=impl, heads={0, 7, H - 1})
 
 
-def test_config5_full_size(device):
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_config5_full_size(device, impl):
     # B=1 H=8 D=128 S=65536 in 8 shards of 8192, causal window 4096, N(0, 0.5^2)
     B, H, D, S, n, W = 1, 8, 128, 65536, 8, 4096
     _full_size_check(device, "C5", B, H, D, S, n, ra.sliding_window_bias(W), 0.5, _causal_rows_t(device, S, W),
-                     _causal_row_np(S, W), heads={0, 3, H - 1})
+                     _causal_row_np(S, W), impl=impl, heads={0, 3, H - 1})
