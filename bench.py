@@ -86,9 +86,9 @@ def pmc_summary(workload, fetch_csv, write_csv):
     f_scale = gib_kib / fetch[pk][0]
     w_scale = gib_kib / write[pk][0]
     out = [f"rocprofv3 HBM byte counters, workload {workload}: one fwd+bwd pass of the ring",
-           "commands (from /tmp, TMPDIR=/tmp, R = repository root), one counter per run:",
-           f"  rocprofv3 --pmc FETCH_SIZE --output-format csv -d $R/gpurun_out/pmc_fetch -o f -- python3 $R/bench.py --workload {workload} --steps 1 --warmup 0 --no-cpu-baseline --no-kernel-timing --copy-probe",
-           f"  rocprofv3 --pmc WRITE_SIZE --output-format csv -d $R/gpurun_out/pmc_write -o w -- python3 $R/bench.py --workload {workload} --steps 1 --warmup 0 --no-cpu-baseline --no-kernel-timing --copy-probe",
+           "commands (from /tmp, TMPDIR=/tmp, R = repository root, OUT = an output directory), one counter per run:",
+           f"  rocprofv3 --pmc FETCH_SIZE --output-format csv -d $OUT/pmc_fetch -o f -- python3 $R/bench.py --workload {workload} --steps 1 --warmup 0 --no-cpu-baseline --no-kernel-timing --copy-probe",
+           f"  rocprofv3 --pmc WRITE_SIZE --output-format csv -d $OUT/pmc_write -o w -- python3 $R/bench.py --workload {workload} --steps 1 --warmup 0 --no-cpu-baseline --no-kernel-timing --copy-probe",
            f"  python3 $R/bench.py --workload {workload} --pmc-summary <f_counter_collection.csv> <w_counter_collection.csv>",
            f"calibration kernel (reads 1 GiB, writes 1 GiB): {pk[:60]}",
            f"  FETCH_SIZE reads {fetch[pk][0]:.0f} KiB -> scale {f_scale:.3f};  WRITE_SIZE reads {write[pk][0]:.0f} KiB -> scale {w_scale:.3f}",

@@ -171,7 +171,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   };
   // the same with B in vector registers
   auto mfma_scores_v = [&](f32x16& acc, const bf16x8& av, const bf16x8& bv) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "v"(bv));
+    // (the B operand was assembled by vector instructions just before: two wait states, which
+    // the compiler would see to for one of its own matrix instructions)
+    asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "v"(bv));
   };
   if (GENERAL && tid < 64) {
     // row l32 of the 32 x 16 operand is [i, i, 1, 1, 0 ...] with i = l32 the query's index in the

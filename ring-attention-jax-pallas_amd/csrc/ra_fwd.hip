@@ -40,18 +40,27 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   __shared__ __attribute__((aligned(16))) int s_seg[4][kKeyTile];
   __shared__ __attribute__((aligned(16))) int s_pre[4][kKeyTile];
   __shared__ unsigned short s_list[GENERAL ? kMaxListTiles : 1];
-  __shared__ unsigned char s_flag[GENERAL ? kMaxListTiles : 1];
+  // The several-shard variants with per-tile terms park a third Q fragment in LDS (s_q2); the
+  // room comes from a one-word stash, from the tile flags sharing the stash's memory (they are
+  // used before a shard's loops, the stash inside them, a barrier separates two shards) and
+  // from a ramp table without its all-zero half.
+  constexpr bool PARK2 = GENERAL && MULTI;
+  __shared__ unsigned char s_flag_own[(GENERAL && !PARK2) ? kMaxListTiles : 1];
   __shared__ int s_red[28];
   __shared__ int s_st[GENERAL ? 8 : 1][12];  // per wave and stretch: first iteration, end, tile_base
-  __shared__ int s_stash[GENERAL ? 3 : 1][GENERAL ? kFwdThreads : 1];
+  __shared__ int s_stash[GENERAL ? (PARK2 ? 1 : 3) : 1][GENERAL ? kFwdThreads : 1];
+  static_assert(!PARK2 || kMaxListTiles <= kFwdThreads * 4, "the tile flags fit the stash");
+  unsigned char* const s_flag = PARK2 ? (unsigned char*)&s_stash[0][0] : s_flag_own;
   // The GENERAL and MULTI variants are a few registers short in their straight-line loop: the
   // first operand fragment of Q waits here and is fetched once per iteration instead.
   constexpr bool TIGHT = GENERAL || MULTI;
   __shared__ __attribute__((aligned(16))) bf16x8 s_q0[TIGHT ? kFwdThreads : 1];
   __shared__ __attribute__((aligned(16))) bf16x8 s_q1[GENERAL ? kFwdThreads : 1];  // the second one too
+  __shared__ __attribute__((aligned(16))) bf16x8 s_q2[PARK2 ? kFwdThreads : 1];    // ... and the third
   // ALiBi inside the straight-line loop (see plain_iteration): the key-side operand of the extra
   // matrix instruction, one fragment per 32-key block and lane
-  __shared__ __attribute__((aligned(16))) bf16x8 s_ramp[GENERAL ? 2 : 1][GENERAL ? 64 : 1];
+  // (lanes 32..63 hold the zero half of the operand: PARK2 gives them one shared zero entry, the last)
+  __shared__ __attribute__((aligned(16))) bf16x8 s_ramp[GENERAL ? (PARK2 ? 65 : 128) : 1];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = tid >> 6;
@@ -85,6 +94,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     for (int s = 0; s < KS; ++s) qf[s] = *(const bf16x8*)(qp + 16 * s);
     if (TIGHT) s_q0[tid] = qf[0];
     if (GENERAL) s_q1[tid] = qf[1];
+    if (PARK2) s_q2[tid] = qf[2];
     if (GENERAL && tid < 64) {
       // row (32 kb + l32) of the 32 x 16 operand is [j, j, 1, 1, 0 ...] with j the key's index in
       // the tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
@@ -97,7 +107,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
           rf[0] = rf[1] = (bf16_t)(float)(32 * kb + l32);
           rf[2] = rf[3] = (bf16_t)1.0f;
         }
-        s_ramp[kb][tid] = rf;
+        if (!PARK2) s_ramp[64 * kb + tid] = rf;
+        else if (tid < 32) s_ramp[32 * kb + tid] = rf;
+        else if (tid == 32 && kb == 0) s_ramp[64] = rf;  // all zero
       }
     }
   }
@@ -879,8 +891,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         f32x16 z;
 #pragma unroll
         for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        SN[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[0][ramp_lane], bq, z, 0, 0, 0);
-        SN[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[1][ramp_lane], bq, z, 0, 0, 0);
+        const int r0 = PARK2 ? (ramp_lane < 32 ? ramp_lane : 64) : ramp_lane;
+        const int r1 = PARK2 ? (ramp_lane < 32 ? 32 + ramp_lane : 64) : 64 + ramp_lane;
+        SN[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[r0], bq, z, 0, 0, 0);
+        SN[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(s_ramp[r1], bq, z, 0, 0, 0);
       } else {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -894,12 +908,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       if (TIGHT) q0 = s_q0[tid];
       bf16x8 q1 = qf[1];
       if (GENERAL) q1 = s_q1[tid];
+      bf16x8 q2 = qf[2];
+      if (PARK2) q2 = s_q2[tid];
       links_of_slot(-1);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int op = 0; op < NOPA; ++op) {
         if (op + PF < NOPA) fr[op + PF] = s_op_frag(kt, op + PF);
-        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? q0 : (op < 4 ? q1 : qf[op >> 1]), SN[op & 1], 0, 0, 0);
+        SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? q0 : (op < 4 ? q1 : (op < 6 ? q2 : qf[op >> 1])), SN[op & 1], 0, 0, 0);
         if (op == NOPA / 4) global_to_lds16_s(k_run, k_voff[0], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES);
         if (NLD == 2 && op == NOPA * 3 / 4)
           global_to_lds16_s(k_run + k_part, k_voff[NLD - 1], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES + RPI * (D * 2));
@@ -1005,8 +1021,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     // it has no register to spare
     if (GENERAL) {
       s_stash[0][tid] = q_seg;
-      s_stash[1][tid] = q_pre;
-      s_stash[2][tid] = __float_as_int(slope2);
+      if (!PARK2) {
+        s_stash[1][tid] = q_pre;
+        s_stash[2][tid] = __float_as_int(slope2);
+      }
       seg_r = pre_r = 0;  // already stored
     }
     for (; i + 4 <= p_end; i += 4) {
@@ -1017,8 +1035,13 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
     if (GENERAL) {
       q_seg = s_stash[0][tid];
-      q_pre = s_stash[1][tid];
-      slope2 = __int_as_float(s_stash[2][tid]);
+      if (!PARK2) {
+        q_pre = s_stash[1][tid];
+        slope2 = __int_as_float(s_stash[2][tid]);
+      } else {
+        q_pre = 0;  // a stretch implies that there is no prefix term: the flag was never loaded
+        slope2 = (flags & RA_BIAS_ALIBI) ? bs.slopes[h] * kLog2e : 0.f;
+      }
     }
     if (GENERAL && seg_on) {
       // the scores of tile i, which the next generic iteration turns into probabilities, came
