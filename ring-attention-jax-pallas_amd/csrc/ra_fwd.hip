@@ -45,6 +45,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // used before a shard's loops, the stash inside them, a barrier separates two shards) and
   // from a ramp table without its all-zero half.
   constexpr bool PARK2 = GENERAL && MULTI;
+  constexpr bool DEFER = GENERAL && MULTI;  // see the end of `iteration`
   __shared__ unsigned char s_flag_own[(GENERAL && !PARK2) ? kMaxListTiles : 1];
   __shared__ int s_red[28];
   __shared__ int s_st[GENERAL ? 8 : 1][12];  // per wave and stretch: first iteration, end, tile_base
@@ -357,11 +358,20 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (j < n && t < NLD) {
       const int k0 = tile_at(j, sb_unused) * kKeyTile;
       issue_part(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + (j & 3) * TILE_BYTES + wave_u * 8 * (D * 2), t);
-      if (GENERAL && t == 0 && tid < kKeyTile) {
+      if (GENERAL && !DEFER && t == 0 && tid < kKeyTile) {
         int kk = min(k0 + tid, a.Lk - 1);
         if (kv_seg) seg_r = kv_seg[kk];
         if (kv_pre) pre_r = kv_pre[kk];
       }
+    }
+  };
+  // the ids of K tile ordinal j, into registers (store_ids publishes them), where they do not
+  // travel with the request
+  auto fetch_ids = [&](int j) {
+    if (j < n && tid < kKeyTile) {
+      const int kk = min(tile_at(j, sb_unused) * kKeyTile + tid, a.Lk - 1);
+      if (kv_seg) seg_r = kv_seg[kk];
+      if (kv_pre) pre_r = kv_pre[kk];
     }
   };
   auto request_v = [&](int j, int t) {
@@ -667,8 +677,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         for (int op = 0; op < 2 * KS; ++op) {
           if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
           SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
-          if (op == (2 * KS) / 4) request_k(i + 3, 0);
-          if (op == (2 * KS) * 3 / 4) request_k(i + 3, 1);
+          if constexpr (!DEFER) {
+            if (op == (2 * KS) / 4) request_k(i + 3, 0);
+            if (op == (2 * KS) * 3 / 4) request_k(i + 3, 1);
+          }
 #pragma unroll
           for (int e = 0; e < EPO; e += 2) {
             const int el = op * EPO + e;  // 0..31 over (kb, r)
@@ -707,8 +719,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         for (int op = 0; op < 4 * DB; ++op) {
           if (op + PF < 4 * DB) fr[op + PF] = pv_op_frag(vt, op + PF);
           oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], pfrag[op / DB], oacc[op % DB], 0, 0, 0);
-          if (op == (4 * DB) / 4) request_v(i + v_ahead, 0);
-          if (op == (4 * DB) * 3 / 4) request_v(i + v_ahead, 1);
+          if constexpr (!DEFER) {
+            if (op == (4 * DB) / 4) request_v(i + v_ahead, 0);
+            if (op == (4 * DB) * 3 / 4) request_v(i + v_ahead, 1);
+          }
 #pragma unroll
           for (int e = 0; e < EPO; e += 2) {
             const int el = op * EPO + e;  // one three-operand maximum per pair of scores
@@ -721,8 +735,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       }
     } else {
       // ---- generic path (first / last / masked / biased tiles): same work, not interleaved -----
-      request_k(i + 3, 0);
-      request_k(i + 3, 1);
+      if constexpr (!DEFER) {
+        request_k(i + 3, 0);
+        request_k(i + 3, 1);
+      }
       if (nxt_valid) compute_s(SN, kt);
       if (cur_valid) {
         float rs = 0.f;
@@ -750,13 +766,27 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
           }
       }
       if (late_half) sync(i + 1);
-      request_v(i + v_ahead, 0);
-      request_v(i + v_ahead, 1);
+      if constexpr (!DEFER) {
+        request_v(i + v_ahead, 0);
+        request_v(i + v_ahead, 1);
+      }
       if (cur_valid) compute_pv(pfrag, vt);
       if (nxt_valid && !nxt_biased) nxt_mx = raw_rowmax(SN);
     }
     if (nxt_biased) nxt_mx = prepare(SN, nkt0, nsegbit, ncls, (i + 1) & 3);
-    if (i + 3 < n) store_ids((i + 3) & 3);
+    if constexpr (DEFER) {
+      // These variants hold part of their state in scratch memory, and a reload waits for every
+      // load issued before it: a generic iteration's requests go out last, behind the ids (plain
+      // loads, awaited by the store), so that nothing in it waits for them.
+      fetch_ids(i + 3);
+      if (i + 3 < n) store_ids((i + 3) & 3);
+      request_k(i + 3, 0);
+      request_k(i + 3, 1);
+      request_v(i + v_ahead, 0);
+      request_v(i + v_ahead, 1);
+    } else {
+      if (i + 3 < n) store_ids((i + 3) & 3);
+    }
     cur_valid = nxt_valid;
     cur_mx = nxt_mx;
   };
