@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // room comes from a one-word stash, from the tile flags sharing the stash's memory (they are
   // used before a shard's loops, the stash inside them, a barrier separates two shards) and
   // from a ramp table without its all-zero half.
-  constexpr bool PARK2 = GENERAL && MULTI;
+  constexpr bool PARK2 = GENERAL;
   constexpr bool DEFER = GENERAL && MULTI;  // see the end of `iteration`
   __shared__ unsigned char s_flag_own[(GENERAL && !PARK2) ? kMaxListTiles : 1];
   __shared__ int s_red[28];
@@ -476,11 +476,19 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
 #pragma unroll
     for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
+    // the fragments that the per-tile-term variants park in LDS are fetched from there here too:
+    // they occupy no register outside the prologue
+    bf16x8 qp0 = qf[0], qp1 = qf[1], qp2 = qf[2];
+    if constexpr (GENERAL) {
+      qp0 = s_q0[tid];
+      qp1 = s_q1[tid];
+    }
+    if constexpr (PARK2) qp2 = s_q2[tid];
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
-      S[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], S[op & 1], 0, 0, 0);
+      S[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? qp0 : (op < 4 ? qp1 : (op < 6 ? qp2 : qf[op >> 1])), S[op & 1], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -671,12 +679,18 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         }
 #pragma unroll
         for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
+        bf16x8 qp0 = qf[0], qp1 = qf[1], qp2 = qf[2];  // from LDS where they are parked there
+        if constexpr (GENERAL) {
+          qp0 = s_q0[tid];
+          qp1 = s_q1[tid];
+        }
+        if constexpr (PARK2) qp2 = s_q2[tid];
         __builtin_amdgcn_sched_barrier(0);
         constexpr int EPO = 32 / (2 * KS);  // score elements converted per MFMA
 #pragma unroll
         for (int op = 0; op < 2 * KS; ++op) {
           if (op + PF < 2 * KS) fr[op + PF] = s_op_frag(kt, op + PF);
-          SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], SN[op & 1], 0, 0, 0);
+          SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? qp0 : (op < 4 ? qp1 : (op < 6 ? qp2 : qf[op >> 1])), SN[op & 1], 0, 0, 0);
           if constexpr (!DEFER) {
             if (op == (2 * KS) / 4) request_k(i + 3, 0);
             if (op == (2 * KS) * 3 / 4) request_k(i + 3, 1);
