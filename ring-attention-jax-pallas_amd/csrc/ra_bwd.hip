@@ -1356,12 +1356,20 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     }
 #pragma unroll
     for (int op = 0; op < PF; ++op) fr[op] = nat_frag((op & 1) ? vt : kt, op >> 1);
+    // the fragments that the per-tile-term variants park in LDS are fetched from there here too:
+    // they occupy no register outside the prologue
+    bf16x8 qp0 = qf[0], qp1 = qf[1], dp0 = dof[0];
+    if constexpr (GENERAL) {
+      qp0 = s_q0[tid];
+      qp1 = s_q1[tid];
+      dp0 = s_do0[tid];
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PF < 2 * KS) fr[op + PF] = nat_frag(((op + PF) & 1) ? vt : kt, (op + PF) >> 1);
-      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], dof[op >> 1], P, 0, 0, 0);
-      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], qf[op >> 1], S, 0, 0, 0);
+      if (op & 1) P = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op == 1 ? dp0 : dof[op >> 1], P, 0, 0, 0);
+      else S = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op == 0 ? qp0 : (op == 2 ? qp1 : qf[op >> 1]), S, 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
