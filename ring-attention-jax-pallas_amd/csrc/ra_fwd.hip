@@ -627,7 +627,13 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     // this wave's share of K_{k+1}, V_k is in LDS once only the requests of barrier k-1 (K_{k+2},
     // V_{k+1}, NLD load instructions each, where they exist) are in flight
     const int pending = (k + 2 < n ? NLD : 0) + (k + 1 < n ? NLD : 0);
-    if (GENERAL || k == 0 || pending == 0) __builtin_amdgcn_s_waitcnt(0x0f70);
+    // The per-tile-term variants fetch ids with ordinary loads, which the compiler awaits without
+    // knowing of the tile loads around them: they wait for everything - except the early waves of
+    // the variants whose generic iterations issue their requests last (DEFER): there the ids are
+    // stored before the requests go out, so at this point only tile loads are in flight and the
+    // most recent ones are, as in the plain case, those of K_{k+2} and V_{k+1}.
+    const bool counted = !GENERAL || (DEFER && !late_half);
+    if (!counted || k == 0 || pending == 0) __builtin_amdgcn_s_waitcnt(0x0f70);
     else if (pending == NLD) __builtin_amdgcn_s_waitcnt(0x0f70 | NLD);
     else __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));
     __syncthreads();
