@@ -45,7 +45,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // used before a shard's loops, the stash inside them, a barrier separates two shards) and
   // from a ramp table without its all-zero half.
   constexpr bool PARK2 = GENERAL;
-  constexpr bool DEFER = GENERAL && MULTI;  // see the end of `iteration`
+  constexpr bool DEFER = GENERAL;  // see the end of `iteration`
   __shared__ unsigned char s_flag_own[(GENERAL && !PARK2) ? kMaxListTiles : 1];
   __shared__ int s_red[28];
   __shared__ int s_st[GENERAL ? 8 : 1][12];  // per wave and stretch: first iteration, end, tile_base
