@@ -520,7 +520,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
                  min(kw + l32, a.Lk - 1);
       tb.dense_vs = bs.dense_sq;
     }
-    apply_bias<false, DENSE>(S, tb, rel0, k_seg, k_pre, ids + 2 * kQTile, ids + 3 * kQTile);
+    apply_bias<false, DENSE, GENERAL>(S, tb, rel0, k_seg, k_pre, ids + 2 * kQTile, ids + 3 * kQTile);
   };
 
   // ---- prologue: tiles 0, 1, 2 requested, S(0) and dP(0) computed ------------------------------
@@ -1402,7 +1402,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     const int rel0 = (q_off + qi) - (kv_off + var0);
     if (DENSE)
       tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
-    apply_bias<true, DENSE>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
+    apply_bias<true, DENSE, GENERAL>(S, tb, rel0, q_seg, q_pre, &s_seg[ids_buf][4 * g], &s_pre[ids_buf][4 * g]);
   };
 
   // ---- prologue: tiles 0, 1, 2 in flight; S^T(0), dP^T(0) computed ------------------------------

@@ -206,14 +206,50 @@ struct TileBias {
   long long dense_vs;   // its stride along the varying side (1 when the keys vary)
 };
 
-template <bool QFIXED, bool DENSE>
+// Branch-free per element: the uniform `flags` only shape a handful of per-lane constants up
+// front (evaluated per element they cost ~25 instructions per score, three times the softmax
+// itself).  Range limit, causal and window terms are ONE interval [lo, hi] of the element's offset
+// `off` on the varying side (rel = rel0 -+ off is monotonic in it); the prefix term is a second
+// bound that only counts where not both sides carry the prefix flag; a segment test against the
+// lane's own id when there is no segment term compares equal; ALiBi with slope 0 adds nothing.
+// TERMS = false: a kernel variant that knows causal / window terms only (the rest compiles away).
+template <bool QFIXED, bool DENSE, bool TERMS>
 RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, int fixed_pre,
                        const int* var_seg, const int* var_pre) {
+  constexpr int kFar = 1 << 29;
+  // one value per wave (a block belongs to one wave's rows and one tile): say so, or the compiler
+  // carries every flag test as a lane mask
+  int flags = __builtin_amdgcn_readfirstlane(tb.flags);
+  if (!TERMS) flags &= RA_BIAS_CAUSAL | RA_BIAS_WINDOW;
+  const bool causal = flags & RA_BIAS_CAUSAL, window = flags & RA_BIAS_WINDOW;
+  const bool segment = flags & RA_BIAS_SEGMENT, prefix = flags & RA_BIAS_PREFIX;
+  int lo = 0, hi = tb.var_limit - 1;  // off >= var_limit: out of range
+  int pre_lo = -kFar, pre_hi = kFar;  // outside [pre_lo, pre_hi]: rel < 0, masked unless both sides are prefix
+  if (QFIXED) {  // rel = rel0 - off: rel < 0 <=> off > rel0, rel >= w <=> off <= rel0 - w, -rel >= w <=> off >= rel0 + w
+    if (causal) hi = min(hi, rel0);
+    if (window) lo = max(lo, rel0 - tb.window + 1);
+    if (window && !causal) hi = min(hi, rel0 + tb.window - 1);
+    if (prefix) pre_hi = rel0;
+  } else {  // rel = rel0 + off: rel < 0 <=> off < -rel0, rel >= w <=> off >= w - rel0, -rel >= w <=> off <= -rel0 - w
+    if (causal) lo = max(lo, -rel0);
+    if (window) hi = min(hi, tb.window - 1 - rel0);
+    if (window && !causal) lo = max(lo, 1 - rel0 - tb.window);
+    if (prefix) pre_lo = -rel0;
+  }
+  // off in [lo, hi] <=> (unsigned)(off - lo) <= (unsigned)(hi - lo); an empty interval (hi < lo)
+  // becomes lo = 1 << 30, span = 0: no off in 0..63 passes
+  const bool none = hi < lo;
+  const unsigned nlo = (unsigned)(none ? -(1 << 30) : -lo), span = (unsigned)(none ? 0 : hi - lo);
+  const unsigned pnlo = (unsigned)(-pre_lo), pspan = (unsigned)(pre_hi - pre_lo);
+  const int seg_ref = fixed_seg;
+  const int pre_on = (prefix && fixed_pre != 0) ? -1 : 0;  // all ones where this lane's side carries the flag
+  const float slope = (flags & RA_BIAS_ALIBI) ? -tb.slope2 : 0.f;
+  const float relf0 = (float)rel0;
 #pragma unroll
   for (int bb = 0; bb < 4; ++bb) {
-    i32x4 vs = {0, 0, 0, 0}, vp = {0, 0, 0, 0};
-    if (tb.flags & RA_BIAS_SEGMENT) vs = *(const i32x4*)(var_seg + 8 * bb);
-    if (tb.flags & RA_BIAS_PREFIX) vp = *(const i32x4*)(var_pre + 8 * bb);
+    i32x4 vs = {seg_ref, seg_ref, seg_ref, seg_ref}, vp = {0, 0, 0, 0};
+    if (segment) vs = *(const i32x4*)(var_seg + 8 * bb);
+    if (prefix) vp = *(const i32x4*)(var_pre + 8 * bb);
     float dn[4] = {0.f, 0.f, 0.f, 0.f};
     if (DENSE) {
 #pragma unroll
@@ -225,18 +261,11 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
       const int r = 4 * bb + c;
       const int off = 8 * bb + c;
       // moving along the varying side: keys advance -> rel decreases; queries advance -> rel increases
-      const int rel = QFIXED ? rel0 - off : rel0 + off;
-      float x = t[r];
-      if (tb.flags & RA_BIAS_ALIBI) x = fmaf(fabsf((float)rel), -tb.slope2, x);
+      const float relf = QFIXED ? relf0 - (float)off : relf0 + (float)off;
+      float x = fmaf(fabsf(relf), slope, t[r]);
       if (DENSE) x = fmaf(dn[c], tb.dense_mul, x);
-      bool msk = off >= tb.var_limit;
-      if (tb.flags & RA_BIAS_CAUSAL) msk |= rel < 0;
-      if (tb.flags & RA_BIAS_WINDOW) {
-        msk |= rel >= tb.window;
-        if (!(tb.flags & RA_BIAS_CAUSAL)) msk |= -rel >= tb.window;
-      }
-      if (tb.flags & RA_BIAS_SEGMENT) msk |= vs[c] != fixed_seg;
-      if (tb.flags & RA_BIAS_PREFIX) msk |= !(((vp[c] != 0) & (fixed_pre != 0)) | (rel >= 0));
+      bool msk = ((unsigned)off + nlo > span) | (vs[c] != seg_ref);
+      msk |= ((unsigned)off + pnlo > pspan) & ((vp[c] & pre_on) == 0);
       t[r] = msk ? RA_NEG_INF : x;
     }
   }

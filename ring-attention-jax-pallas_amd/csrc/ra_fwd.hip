@@ -541,7 +541,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       const int rel0 = (q_off + qi) - (kv_off + var0);
       if (DENSE)
         tb.dense = dense_ptr + b * bs.dense_sb + h * bs.dense_sh + (long long)min(qi, a.Lq - 1) * bs.dense_sq + var0;
-      apply_bias<true, DENSE>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
+      apply_bias<true, DENSE, GENERAL>(S[kb], tb, rel0, q_seg, q_pre, &s_seg[ids_buf][32 * kb + 4 * g],
                        &s_pre[ids_buf][32 * kb + 4 * g]);
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
