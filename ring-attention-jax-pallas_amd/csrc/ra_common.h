@@ -243,32 +243,48 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
   const unsigned pnlo = (unsigned)(-pre_lo), pspan = (unsigned)(pre_hi - pre_lo);
   const int seg_ref = fixed_seg;
   const int pre_on = (prefix && fixed_pre != 0) ? -1 : 0;  // all ones where this lane's side carries the flag
-  const float slope = (flags & RA_BIAS_ALIBI) ? -tb.slope2 : 0.f;
+  const float slope = -tb.slope2;
   const float relf0 = (float)rel0;
+  // The two terms that cost the most per element, ALiBi (two instructions) and prefix (six), get
+  // code of their own, chosen once per block by a uniform branch.
+  auto body = [&](auto with_alibi, auto with_prefix) {
+    constexpr bool ALI = decltype(with_alibi)::value, PRE = decltype(with_prefix)::value;
 #pragma unroll
-  for (int bb = 0; bb < 4; ++bb) {
-    i32x4 vs = {seg_ref, seg_ref, seg_ref, seg_ref}, vp = {0, 0, 0, 0};
-    if (segment) vs = *(const i32x4*)(var_seg + 8 * bb);
-    if (prefix) vp = *(const i32x4*)(var_pre + 8 * bb);
-    float dn[4] = {0.f, 0.f, 0.f, 0.f};
-    if (DENSE) {
+    for (int bb = 0; bb < 4; ++bb) {
+      i32x4 vs = {seg_ref, seg_ref, seg_ref, seg_ref}, vp = {0, 0, 0, 0};
+      if (segment) vs = *(const i32x4*)(var_seg + 8 * bb);
+      if (PRE) vp = *(const i32x4*)(var_pre + 8 * bb);
+      float dn[4] = {0.f, 0.f, 0.f, 0.f};
+      if (DENSE) {
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        if (8 * bb + c < tb.var_limit) dn[c] = QFIXED ? tb.dense[8 * bb + c] : tb.dense[(8 * bb + c) * tb.dense_vs];
+        for (int c = 0; c < 4; ++c)
+          if (8 * bb + c < tb.var_limit) dn[c] = QFIXED ? tb.dense[8 * bb + c] : tb.dense[(8 * bb + c) * tb.dense_vs];
+      }
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int r = 4 * bb + c;
+        const int off = 8 * bb + c;
+        float x = t[r];
+        if (ALI) {
+          // moving along the varying side: keys advance -> rel decreases; queries advance -> rel increases
+          const float relf = QFIXED ? relf0 - (float)off : relf0 + (float)off;
+          x = fmaf(fabsf(relf), slope, x);
+        }
+        if (DENSE) x = fmaf(dn[c], tb.dense_mul, x);
+        bool msk = ((unsigned)off + nlo > span) | (vs[c] != seg_ref);
+        if (PRE) msk |= ((unsigned)off + pnlo > pspan) & ((vp[c] & pre_on) == 0);
+        t[r] = msk ? RA_NEG_INF : x;
+      }
     }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const int r = 4 * bb + c;
-      const int off = 8 * bb + c;
-      // moving along the varying side: keys advance -> rel decreases; queries advance -> rel increases
-      const float relf = QFIXED ? relf0 - (float)off : relf0 + (float)off;
-      float x = fmaf(fabsf(relf), slope, t[r]);
-      if (DENSE) x = fmaf(dn[c], tb.dense_mul, x);
-      bool msk = ((unsigned)off + nlo > span) | (vs[c] != seg_ref);
-      msk |= ((unsigned)off + pnlo > pspan) & ((vp[c] & pre_on) == 0);
-      t[r] = msk ? RA_NEG_INF : x;
-    }
-  }
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  const bool alibi = flags & RA_BIAS_ALIBI;
+  if (!TERMS) body(No{}, No{});
+  else if (alibi && prefix) body(Yes{}, Yes{});
+  else if (alibi) body(Yes{}, No{});
+  else if (prefix) body(No{}, Yes{});
+  else body(No{}, No{});
 }
 
 // Positional classification of a rectangle of scores: queries [qlo, qhi], keys [klo, khi]
