@@ -54,6 +54,11 @@ extern "C" {
 #define RA_BIAS_PREFIX 8   /* (q_prefix & kv_prefix) | kv_pos <= q_pos (ring.py:399-406)    */
 #define RA_BIAS_ALIBI 16   /* additive -slope[h] * |q_pos - kv_pos|                       */
 #define RA_BIAS_DENSE 32   /* additive fp32 block, the array a bias_fn returns (ring.py:107) */
+/* With RA_BIAS_SEGMENT one call takes shards of at most this many tokens (the kernels sort a
+ * shard's tiles by id range into a list of that capacity); RA_ERR_SHAPE beyond.  A longer shard
+ * is walked as several shorter ones: the block step is associative over key/value shards and
+ * independent over query rows (ring.py:58-76). */
+#define RA_MAX_SEGMENT_SHARD 65536
 
 #define RA_DTYPE_BF16 0
 #define RA_DTYPE_F32 1

@@ -59,6 +59,24 @@ def _axis_size(axis_name) -> int:
     raise TypeError("axis_name must be a RingAxis, an int ring size or a (name, size) pair")
 
 
+def _walked_ring_size(n: int, Sq: int, Sk: int, bias_fn) -> int:
+    """Ring size that the emulation walks.  Under a segment bias one call of the library takes
+    shards of at most ``RA_MAX_SEGMENT_SHARD`` tokens; a ring whose shards are longer is walked as
+    a finer ring (every shard cut into f equal pieces).  The online softmax is associative over
+    key/value shards and independent over query rows (ring.py:58-76), so the result is the same
+    up to the rounding of a different summation order.  Lengths that no f <= 4096 divides keep
+    ``n`` (and the library reports the limit)."""
+    if not (isinstance(bias_fn, BiasFn) and bias_fn.segments) or Sq % n or Sk % n:
+        return n
+    longest = max(Sq // n, Sk // n)
+    if longest <= _lib.RA_MAX_SEGMENT_SHARD:
+        return n
+    for f in range(-(-longest // _lib.RA_MAX_SEGMENT_SHARD), 4097):
+        if (Sq // n) % f == 0 and (Sk // n) % f == 0:
+            return n * f
+    return n
+
+
 def _stream() -> C.c_void_p:
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -700,13 +718,14 @@ def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable,
         pad = (0, d_pad - d_true)
         q, k, v = (torch.nn.functional.pad(x, pad) for x in (q, k, v))
     q, k, v = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
-    plan = _RingPlan(q, k, n, bias_fn, bias_q_kwargs, bias_kv_kwargs)
+    plan = _RingPlan(q, k, _walked_ring_size(n, q.shape[1], k.shape[1], bias_fn), bias_fn, bias_q_kwargs,
+                     bias_kv_kwargs)
     out, lse = _RingAttentionFn.apply(q, k, v, plan, float(sm_scale), out_dtype, block_impl == "hip_fused")
     if d_pad != d_true:
         out = out[..., :d_true]
     if in_dtype not in (torch.float32, torch.bfloat16):
         out = out.to(in_dtype)
-    lse_full = lse.permute(1, 2, 0, 3).reshape(plan.B, plan.H, n * plan.Lq)
+    lse_full = lse.permute(1, 2, 0, 3).reshape(plan.B, plan.H, plan.n * plan.Lq)
     return out, lse_full
 
 

@@ -1041,3 +1041,24 @@ def test_config5_full_size(device, impl):
     B, H, D, S, n, W = 1, 8, 128, 65536, 8, 4096
     _full_size_check(device, "C5", B, H, D, S, n, ra.sliding_window_bias(W), 0.5, _causal_rows_t(device, S, W),
                      _causal_row_np(S, W), impl=impl, heads={0, 3, H - 1})
+
+
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_segment_shards_longer_than_one_call_takes(device, impl):
+    # one "device" holding 98304 tokens of three documents, causal: above the 65536 tokens that a
+    # call takes under a segment bias, so the ring is walked as two shards of 49152
+    B, H, D, S, n = 1, 2, 64, 98304, 1
+    seg = np.zeros((B, S), np.int32)
+    seg[0, 30000:] += 1
+    seg[0, 70001:] += 1
+    tseg = torch.from_numpy(seg).to(device)
+    tpos = torch.arange(S, device=device)
+    pos = np.arange(S)
+
+    def rows_t(b, h, i0, i1):
+        ok = (tseg[b, i0:i1, None] == tseg[b, None, :]) & (tpos[None, :] <= tpos[i0:i1, None])
+        return torch.where(ok, 0.0, -torch.inf).double()
+
+    brow = lambda b, h, i: np.where((seg[b] == seg[b, i]) & (pos <= i), 0.0, -np.inf)
+    _full_size_check(device, "long segment shard", B, H, D, S, n, ra.segment_bias() + ra.causal_bias(), 1.0, rows_t,
+                     brow, {"q_segment_ids": tseg}, {"kv_segment_ids": tseg}, impl=impl, n_rows=64)

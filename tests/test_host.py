@@ -55,6 +55,21 @@ def test_ring_self_attention_argument_rules():
         ra.ring_self_attention(q, q, q, 2, prefix_mask=pos)  # ring.py:373
 
 
+def test_long_segment_shards_are_walked_as_a_finer_ring():
+    seg, causal = ra.segment_bias(), ra.causal_bias()
+    cap = rr._lib.RA_MAX_SEGMENT_SHARD
+    assert cap == 65536
+    assert rr._walked_ring_size(1, 98304, 98304, seg + causal) == 2      # 2 x 49152
+    assert rr._walked_ring_size(2, 4 * cap, 4 * cap, seg) == 4           # shards of 2 x cap -> cap
+    assert rr._walked_ring_size(2, 4 * cap + 6, 4 * cap + 6, seg) == 10  # shards of 131075 = 5 x 26215
+    assert rr._walked_ring_size(1, 98304, 1024, seg) == 2                # the longer side decides
+    assert rr._walked_ring_size(1, 98304, 1023, seg) == 3                # ... and both must divide
+    assert rr._walked_ring_size(8, 8 * cap, 8 * cap, seg) == 8           # at the limit: untouched
+    assert rr._walked_ring_size(1, 98304, 98304, causal) == 1            # no segment term: no limit
+    assert rr._walked_ring_size(1, 98304, 98304, None) == 1
+    assert rr._walked_ring_size(1, 2 * 65537, 2 * 65537, seg) == 1       # 2 x a prime: left to the library's check
+
+
 def test_ring_plan_shards_and_offsets():
     q = torch.zeros(2, 64, 2, 64, dtype=torch.bfloat16)
     k = torch.zeros(2, 32, 2, 64, dtype=torch.bfloat16)
