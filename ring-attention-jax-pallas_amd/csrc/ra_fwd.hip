@@ -17,7 +17,6 @@ constexpr int kFwdThreads = 512;
 constexpr int kFwdRows = 256;   // query rows per workgroup
 constexpr int kKeyTile = 64;    // keys per LDS tile
 constexpr int kMaxListTiles = 1024;
-constexpr int kPlainMinTiles = 16;  // shortest stretch of plain tiles that takes the straight-line loop
 
 // MULTI: grid dimension y is a ring pass, the trip of one query shard around the ring.  The launch
 // walks the key/value shards that `ring` lists for the pass one after another (the arguments of
@@ -125,12 +124,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // whole-ring launch: no carry comes in, the finished output goes out
   float m_run = WHOLE ? RA_NEG_INF : pass_m()[row] * kLog2e;  // exponent reference (log2 domain), moves lazily
   float l_run = 0.f, lr_run = 0.f;  // per-lane partial sums (this lane's keys only)
-  // In a long stretch of completely unmasked tiles (at least kPlainMinTiles of them) a tile adds
-  // only its ROUNDED probabilities, to this third sum, which counts for both l and lr: the
-  // rounding errors of the thousand or more terms are unbiased and their sum moves the logsumexp
-  // by a few 1e-5, far less than its tolerance, and the row sums cost one dot instruction per
-  // pair of scores instead of three additions.
-  float lp_run = 0.f;
+  // (Both sums in every loop: where a row's weight sits on one or two keys, the rounded sum
+  // alone carries the rounding error of those few weights, up to 2^-8 relative, into the
+  // logsumexp.)
   f32x16 oacc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -560,7 +556,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       m_run = m_new;
       l_run *= corr;
       lr_run *= corr;
-      lp_run *= corr;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -897,16 +892,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       pw[w >> 2][w & 3] = pk[w];
     };
     auto link4 = [&](int w) {
-      if constexpr (GENERAL) {
-        // both sums: under ALiBi or inside a short document a row's weight sits on a few keys,
-        // and the rounding of those few terms alone would move the logsumexp by up to 2e-3
-        lr_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lr_run, false);
-        l_run += e[w][0] + e[w][1];
-        asm volatile("" : "+v"(lr_run), "+v"(l_run));
-      } else {
-        lp_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lp_run, false);
-        asm volatile("" : "+v"(lp_run));
-      }
+      lr_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lr_run, false);
+      l_run += e[w][0] + e[w][1];
+      asm volatile("" : "+v"(lr_run), "+v"(l_run));
     };
     auto links_of_slot = [&](int gs) {
 #pragma unroll
@@ -1021,9 +1009,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   if constexpr (!GENERAL) {
     // one stretch; iteration i is plain for st_lo[0] <= i < plain_end
     const int plain_end =
-        __builtin_amdgcn_readfirstlane(st_hi[0] - st_lo[0] < kPlainMinTiles
-                                           ? 0
-                                           : min(min(st_hi[0] - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));
+        __builtin_amdgcn_readfirstlane(min(min(st_hi[0] - 1, run_hi - 3), a.Lk / kKeyTile - tile_base - 3));
     for (; i < n && !(i >= st_lo[0] && i + 4 <= plain_end); i += 4) {
       iteration(P0{}, i, sa, sb);
       if (i + 1 < n) iteration(P1{}, i + 1, sb, sa);
@@ -1126,14 +1112,14 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // A wave that gathered no probability mass (no tile listed for its workgroup, or every score
   // masked) has nothing to merge: with l_step = 0 and an unchanged maximum the merge below is the
   // identity, so the carry's 32 rows stay where they are, unread.
-  if (!WHOLE && __all(l_run == 0.f && lr_run == 0.f && lp_run == 0.f)) return;
+  if (!WHOLE && __all(l_run == 0.f && lr_run == 0.f)) return;
   if constexpr (WHOLE) {
     {
       // out = o_step / (sum of the rounded weights): the normalised average of V;
       // lse = ln 2 (m_run + log2 l_step) with the exact sum.  A row that saw no key: 0 / 0 and -inf.
       const int qi_out = q0 + wave * 32 + l32;
       row = ((long long)b * a.H + h) * a.Lq + min(qi_out, a.Lq - 1);
-      const float l_step = half_sum(l_run + lp_run), lr_step = half_sum(lr_run + lp_run);
+      const float l_step = half_sum(l_run), lr_step = half_sum(lr_run);
       const float inv = 1.0f / lr_step;
       if (q_valid) {
         const long long at = b * a.out_sb + h * a.out_sh + (long long)qi_out * a.out_sl + 4 * g;
@@ -1173,7 +1159,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     // over the whole loop
     row = ((long long)b * a.H + h) * a.Lq + min(q0 + wave * 32 + l32, a.Lq - 1);
     const float m_in = pass_m()[row] * kLog2e;
-    const float l_step = half_sum(l_run + lp_run), lr_step = half_sum(lr_run + lp_run);
+    const float l_step = half_sum(l_run), lr_step = half_sum(lr_run);
     const float m_out = m_true;  // started from m_in, so it already covers the carry
     const float m_safe = (m_out == RA_NEG_INF) ? 0.f : m_out;
     const float f_in = fast_exp2(m_in - m_safe);   // 0 for an empty carry
