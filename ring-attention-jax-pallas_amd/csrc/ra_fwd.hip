@@ -855,8 +855,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const unsigned v_dst = v_dst0 + (late_half ? ((PAR + 3) & 3) : ((PAR + 2) & 3)) * TILE_BYTES;
     // ---- S(i+1) MFMAs, then O += P(i) V_i, with the softmax arithmetic of tile i and the row
     // maximum of S(i+1) in their shadow.  The chain of a pair of scores (scale and shift, exp2,
-    // pack, row sum) is spread over four consecutive MFMA slots, one link per slot, so that no
-    // vector instruction waits for the result of the one before it; the sixteen pairs of a lane
+    // pack, rounded row sum, exact row sum) is spread over five consecutive MFMA slots, one link
+    // per slot, so that no vector instruction waits for the result of the one before it and no
+    // slot carries both the exp2 pair of one chain and all three sum instructions of another
+    // (1.8 % of the kernel); the sixteen pairs of a lane
     // are spread over both MFMA blocks so that every slot carries about the same vector work:
     // half of them (the first two operand fragments of P) in the score block, the other half in
     // the first three quarters of the output block, the row maxima in the slots that remain.
@@ -893,8 +895,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     };
     auto link4 = [&](int w) {
       lr_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk[w]), ones2, lr_run, false);
+      asm volatile("" : "+v"(lr_run));
+    };
+    auto link5 = [&](int w) {
       l_run += e[w][0] + e[w][1];
-      asm volatile("" : "+v"(lr_run), "+v"(l_run));
+      asm volatile("" : "+v"(l_run));
     };
     auto links_of_slot = [&](int gs) {
 #pragma unroll
@@ -903,6 +908,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         if (slot_of(w) == gs) link2(w);
         if (slot_of(w) + 1 == gs) link3(w);
         if (slot_of(w) + 2 == gs) link4(w);
+        if (slot_of(w) + 3 == gs) link5(w);
       }
     };
     {
