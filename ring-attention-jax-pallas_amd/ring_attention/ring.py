@@ -25,6 +25,7 @@ succeeds but every call raises.
 """
 from __future__ import annotations
 
+import collections
 import ctypes as C
 import math
 from dataclasses import dataclass
@@ -35,11 +36,29 @@ import torch
 from . import _lib
 from .bias import BiasFn, BlockBias
 
-# "hip": one launch per ring step, the reference's loop; "pallas" is accepted as an alias (the
-# fused-kernel choice there).  "hip_fused": one launch for ALL ring passes - the kernels walk the
-# shards of a query (or key/value) shard's whole trip around the ring themselves, one grid row per
-# resident shard.
-_IMPLS = ("hip", "pallas", "hip_fused")
+# The reference's two values (ring.py:255,296-312) plus the two launch schemes by name:
+#   "pallas"    its default, "fused kernels": the library picks the launch scheme - the whole ring
+#               per launch (below) wherever that applies, a launch per step otherwise;
+#   "jax"       its plain per-block loop: one launch per ring step (the same as "hip");
+#   "hip"       one launch per ring step, the reference's loop (ring.py:104-132) as it stands;
+#   "hip_fused" one launch for ALL ring passes - the kernels walk the shards of a query (or
+#               key/value) shard's whole trip around the ring themselves, one grid row per
+#               resident shard.
+_IMPLS = ("pallas", "jax", "hip", "hip_fused")
+
+
+def _launch_whole_ring(block_impl: str, plan: "_RingPlan") -> bool:
+    """Which launch scheme a call takes.  On one GPU every shard of the emulated ring is resident,
+    so nothing has to wait for a transfer and the whole ring can go into one launch: never slower
+    than a launch per step, and up to twice as fast where one step cannot fill the chip (shards of
+    a few thousand tokens) or where a positional mask leaves a step work for only some of its
+    workgroups.  A callable ``bias_fn`` keeps the launch per step: its dense block is built per
+    (query shard, key/value shard) pair and only one is alive at a time that way."""
+    if block_impl == "hip_fused":
+        return True
+    if block_impl in ("hip", "jax"):
+        return False
+    return plan.callable is None
 
 
 @dataclass(frozen=True)
@@ -489,6 +508,119 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
     return out, lse
 
 
+_PLAN_CACHE: "collections.OrderedDict" = collections.OrderedDict()
+_PLAN_CACHE_SIZE = 8
+
+
+def clear_plan_cache() -> None:
+    """Drop the cached ring plans (and the references to bias arrays that they hold)."""
+    _PLAN_CACHE.clear()
+
+
+def _plan_for(q, k, n, bias_fn, q_kwargs, kv_kwargs) -> "_RingPlan":
+    """The ``_RingPlan`` of a call, from a small cache: a plan (shard offsets read back from the
+    position arrays, id arrays converted to int32, the parameter blocks of the whole-ring
+    launches) depends on shapes, the ring size and the bias arrays only, so a caller who repeats a
+    call - a training loop - pays for it once.  A bias array is identified by the tensor object and
+    its version counter; the cache entry keeps the object alive, so its identity cannot be taken
+    over by another tensor, and an in-place change gives a new version and a new plan."""
+    def ident(t):
+        return (id(t), t._version) if isinstance(t, torch.Tensor) else ("v", t)
+
+    fn_key = bias_fn
+    if isinstance(bias_fn, BiasFn):
+        fn_key = (bias_fn.causal, bias_fn.window, bias_fn.segments, bias_fn.prefix,
+                  None if bias_fn.alibi_slopes is None else ident(bias_fn.alibi_slopes))
+    elif bias_fn is not None:
+        fn_key = ("callable", id(bias_fn))
+    kw_key = tuple(tuple(sorted((a, ident(t)) for a, t in (kw or {}).items())) for kw in (q_kwargs, kv_kwargs))
+    key = (tuple(q.shape), tuple(k.shape), str(q.device), n, fn_key, kw_key)
+    hit = _PLAN_CACHE.get(key)
+    if hit is not None:
+        _PLAN_CACHE.move_to_end(key)
+        return hit[0]
+    plan = _RingPlan(q, k, n, bias_fn, q_kwargs, kv_kwargs)
+    _PLAN_CACHE[key] = (plan, bias_fn, dict(q_kwargs or {}), dict(kv_kwargs or {}))
+    while len(_PLAN_CACHE) > _PLAN_CACHE_SIZE:
+        _PLAN_CACHE.popitem(last=False)
+    return plan
+
+
+# A callable's dense blocks are [b, h | 1, lq, lk] fp32 each: the several-step launches below take
+# as many of them per launch as fit this many bytes (and at most 16, what one launch walks).
+_DENSE_BLOCKS_BYTES = 1 << 30
+
+
+def _row_chunks(plan: "_RingPlan", r: int):
+    """The ring steps of query shard r in ring order, in chunks whose dense blocks are alive
+    together: lists of (key/value shard, BlockBias)."""
+    n = plan.n
+    chunk, used = [], 0
+    for t in range(n):
+        src = (r - t) % n  # ring.py:51-55
+        bias = plan.block_bias(r, src)
+        size = bias.dense.numel() * 4 if bias is not None and bias.dense is not None else 0
+        if chunk and (len(chunk) == 16 or used + size > _DENSE_BLOCKS_BYTES):
+            yield chunk
+            chunk, used = [], 0
+        chunk.append((src, bias))
+        used += size
+    if chunk:
+        yield chunk
+
+
+def _ring_forward_rows(q, k, v, plan: "_RingPlan", sm_scale, out_dtype, timer=_NO_TIMER):
+    """The several-step launch scheme for a callable ``bias_fn``: one query shard at a time, its
+    ring steps in launches of up to 16 (``ra_fwd_steps``, the step's running state in registers
+    between the shards), so that only the dense blocks of one launch are alive."""
+    n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
+    dev = q.device
+    out = torch.empty((B, n * Lq, H, D), dtype=out_dtype, device=dev)
+    lse = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    o, m, l = init_carry(B, H, Lq, D, dev)
+    for r in range(n):
+        if r:
+            reset_carry(o, m, l)
+        qr = _shard_bhld(q, r, Lq)
+        for chunk in _row_chunks(plan, r):
+            with timer.span("fwd_ring", r, -1):
+                fwd_blocks(qr, [(_shard_bhld(k, s, Lk), _shard_bhld(v, s, Lk)) for s, _ in chunk],
+                           [b for _, b in chunk], o, m, l, sm_scale)
+        finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])
+    return out, lse
+
+
+def _ring_backward_rows(q, k, v, out, lse, do, plan: "_RingPlan", sm_scale, timer=_NO_TIMER):
+    """Backward twin of ``_ring_forward_rows``: every dense block is built ONCE and serves both
+    halves of its step - the dQ product of its query shard (one launch per chunk of blocks,
+    ``ra_bwd_dq_steps``) and the dK / dV products of its key/value shard (one launch per block,
+    into that shard's fp32 accumulators)."""
+    n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
+    dev = q.device
+    delta = torch.empty((n, B, H, Lq), dtype=torch.float32, device=dev)
+    for s in range(n):
+        precompute_delta(_shard_bhld(out, s, Lq), _shard_bhld(do, s, Lq), delta[s])
+    dq_acc = torch.empty((B, H, Lq, D), dtype=torch.float32, device=dev)
+    dkv_acc = torch.zeros((2, n, B, H, Lk, D), dtype=torch.float32, device=dev)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    for r in range(n):
+        dq_acc.zero_()
+        qr, dor = _shard_bhld(q, r, Lq), _shard_bhld(do, r, Lq)
+        for chunk in _row_chunks(plan, r):
+            args = [(qr, _shard_bhld(k, s, Lk), _shard_bhld(v, s, Lk), dor, lse[r], delta[r], dq_acc,
+                     dkv_acc[0, s], dkv_acc[1, s], b) for s, b in chunk]
+            with timer.span("bwd_dq_ring", r, -1):
+                _bwd_steps("dq", args, sm_scale)
+            for a in args:
+                with timer.span("bwd_dkdv", r, -1):
+                    _bwd_step(*a, sm_scale, parts=1)
+        _finalize_grad(dq_acc, _shard_bhld(dq, r, Lq))
+    for s in range(n):
+        _finalize_grad(dkv_acc[0, s], _shard_bhld(dk, s, Lk))
+        _finalize_grad(dkv_acc[1, s], _shard_bhld(dv, s, Lk))
+    return dq, dk, dv
+
+
 def _pass_steps(plan: "_RingPlan", cache_key, key, build):
     """The parameter blocks of all ring passes of one kind, built once per plan and set of input
     tensors: only the pointers of buffers allocated per call are patched afterwards."""
@@ -506,6 +638,8 @@ def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO
     launch is everything (ra_fwd_ring: the carry of ring.py:104-132 stays in registers, output and
     logsumexp come out finished); a ring too large for that, or ``whole=False``, takes three
     launches: carry reset, the ring (ra_fwd_passes), finalisation."""
+    if plan.callable is not None:
+        return _ring_forward_rows(q, k, v, plan, sm_scale, out_dtype, timer)
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     lib = _lib.load()
@@ -528,8 +662,6 @@ def _ring_forward_fused(q, k, v, plan: _RingPlan, sm_scale, out_dtype, timer=_NO
 
     key = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(), k.stride(), v.stride(), sm_scale)
     steps, counts, _keep = _pass_steps(plan, "fwd", key, build)
-    if plan.callable is not None:
-        steps, counts, _keep = build()  # a callable's dense blocks are fresh tensors every time
     if whole:
         with timer.span("fwd_ring", -1, -1):
             rc = lib.ra_fwd_ring(steps, counts, n, out.data_ptr(), dt, Lq * ov.stride(2), ov.stride(0), ov.stride(1),
@@ -561,6 +693,8 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
     launches store the finished bf16 gradients themselves (ra_bwd_dkdv_ring, ra_bwd_dq_ring); a
     ring too large for that, or ``whole=False``, adds into zeroed fp32 accumulators
     (ra_bwd_*_passes) that three more launches cast."""
+    if plan.callable is not None:
+        return _ring_backward_rows(q, k, v, out, lse, do, plan, sm_scale, timer)
     n, B, H, D, Lq, Lk = plan.n, plan.B, plan.H, plan.D, plan.Lq, plan.Lk
     dev = q.device
     lib = _lib.load()
@@ -592,8 +726,6 @@ def _ring_backward_fused(q, k, v, out, lse, do, plan: _RingPlan, sm_scale, timer
 
     key = (q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(), k.stride(), v.stride(), do.stride(), sm_scale)
     by_kv, by_q, pairs, counts, _keep = _pass_steps(plan, "bwd", key, build)
-    if plan.callable is not None:
-        by_kv, by_q, pairs, counts, _keep = build()
     s_row = lse[0].numel() * 4
     do_shard = Lq * do.stride(1) * do.element_size()
     for arr, pr in zip((by_kv, by_q), pairs):
@@ -690,7 +822,7 @@ class _RingAttentionFn(torch.autograd.Function):
 
 def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = None, bias_q_kwargs=None,
                             bias_kv_kwargs=None, sm_scale: Optional[float] = None,
-                            block_impl: str = "hip", out_dtype=None):
+                            block_impl: str = "pallas", out_dtype=None):
     """``ring_attention`` that also returns the logsumexp ``[b, h, S]`` (the ``L`` residual of
     ring.py:135)."""
     if block_impl not in _IMPLS:
@@ -718,9 +850,10 @@ def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable,
         pad = (0, d_pad - d_true)
         q, k, v = (torch.nn.functional.pad(x, pad) for x in (q, k, v))
     q, k, v = _kernel_ready(q), _kernel_ready(k), _kernel_ready(v)
-    plan = _RingPlan(q, k, _walked_ring_size(n, q.shape[1], k.shape[1], bias_fn), bias_fn, bias_q_kwargs,
+    plan = _plan_for(q, k, _walked_ring_size(n, q.shape[1], k.shape[1], bias_fn), bias_fn, bias_q_kwargs,
                      bias_kv_kwargs)
-    out, lse = _RingAttentionFn.apply(q, k, v, plan, float(sm_scale), out_dtype, block_impl == "hip_fused")
+    out, lse = _RingAttentionFn.apply(q, k, v, plan, float(sm_scale), out_dtype,
+                                      _launch_whole_ring(block_impl, plan))
     if d_pad != d_true:
         out = out[..., :d_true]
     if in_dtype not in (torch.float32, torch.bfloat16):
@@ -730,7 +863,7 @@ def ring_attention_with_lse(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable,
 
 
 def ring_attention(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = None, bias_q_kwargs=None,
-                   bias_kv_kwargs=None, sm_scale: Optional[float] = None, block_impl: str = "hip"):
+                   bias_kv_kwargs=None, sm_scale: Optional[float] = None, block_impl: str = "pallas"):
     """Ring attention - general (reference ``ring_attention``, ring.py:246-325).
 
     Args:
@@ -744,10 +877,12 @@ def ring_attention(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = 
             for a ``BiasFn``: ``q_segment_ids``, ``q_positions``, ``q_prefix_mask`` and their
             ``kv_`` twins.
         sm_scale: softmax scale, 1/sqrt(d) if unspecified.
-        block_impl: ``"hip"`` (one kernel launch per ring step; ``"pallas"`` is accepted as an
-            alias) or ``"hip_fused"`` (one launch for all ring passes: the kernels walk the shards
-            themselves, which pays when shards are small); anything else raises ``ValueError`` as
-            the reference does (ring.py:312).
+        block_impl: the reference's ``"pallas"`` (its default, ring.py:255: the library picks the
+            launch scheme - the whole ring per launch unless ``bias_fn`` is a callable) and
+            ``"jax"`` (one kernel launch per ring step), or the launch schemes by name: ``"hip"``
+            (launch per step) and ``"hip_fused"`` (one launch for all ring passes: the kernels walk
+            the shards themselves); anything else raises ``ValueError`` as the reference does
+            (ring.py:312).  Every value runs the same kernels on the same bf16 operands.
     Returns:
         attention output ``[b, S, h, d]``; differentiable w.r.t. q, k, v.
     """
@@ -758,7 +893,7 @@ def ring_attention(q, k, v, axis_name, bias_fn: Union[BiasFn, Callable, None] = 
 
 def ring_self_attention(q, k, v, mesh, pspec=None, sm_scale: Optional[float] = None,
                         causal: bool = False, segment_ids=None, positions=None, prefix_mask=None,
-                        block_impl: str = "hip"):
+                        block_impl: str = "pallas"):
     """Ring attention for self-attention (reference ``ring_self_attention``, ring.py:328-449).
 
     Supports full bidirectional attention (default), block-sparse attention via

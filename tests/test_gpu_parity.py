@@ -131,8 +131,17 @@ def test_reference_shapes_self_attention(device, seed, length, h, d):
     assert out.dtype == torch.float32 and out.shape == q.shape
     bias = R.make_bias_fn(causal=True, use_segments=True)(
         q_segment_ids=seg, kv_segment_ids=seg, q_positions=pos, kv_positions=pos)
-    want, _ = R.mha_dense(q, k, v, bias)
-    assert np.abs(out.cpu().numpy() - want).max() <= OUT_TOL
+    want, want_lse = R.mha_dense(q, k, v, bias)
+    got = out.cpu().numpy()
+    assert np.abs(got - want).max() <= OUT_TOL and _out_rel(got, want) <= OUT_REL
+    # the logsumexp of the same call: ring_self_attention is ring_attention with this bias (ring.py:376-449)
+    seg_t, pos_t = _dev(seg, device), _dev(pos, device)
+    out2, lse = ra.ring_attention_with_lse(
+        _dev(q, device), _dev(k, device), _dev(v, device), ra.RingAxis("sp", 8),
+        bias_fn=ra.causal_bias() + ra.segment_bias(), bias_q_kwargs={"q_segment_ids": seg_t, "q_positions": pos_t},
+        bias_kv_kwargs={"kv_segment_ids": seg_t, "kv_positions": pos_t})
+    assert torch.equal(out2, out)
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_TOL
 
 
 # ---- bias functors --------------------------------------------------------------------------------
@@ -775,10 +784,11 @@ def _random_cases(seed, count):
 
 @pytest.mark.parametrize("seed", [0, 1, 2, 3])
 def test_random_configurations(device, seed):
-    """Seeded random shapes and bias combinations, each through both launch schemes, against the
-    dense oracle."""
+    """Seeded random shapes and bias combinations, each through both launch schemes and through the
+    default block_impl (the reference's "pallas": the library picks the scheme), against the dense
+    oracle."""
     for case, kind, kw in _random_cases(seed, 12):
-        for impl in ("hip", "hip_fused"):
+        for impl in ("hip", "hip_fused", "pallas"):
             _check(device, f"random {seed}.{case} {kind}", impl=impl, **kw)
 
 
@@ -1008,11 +1018,12 @@ def test_config2_full_size(device, impl):
                      _causal_row_np(S), impl=impl, n_rows=64)
 
 
-def test_config3_full_size(device):
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_config3_full_size(device, impl):
     # B=1 H=32 D=128 S=131072 in 8 shards of 16384, causal: the benchmark workload
     B, H, D, S, n = 1, 32, 128, 131072, 8
     _full_size_check(device, "C3", B, H, D, S, n, ra.causal_bias(), 1.0, _causal_rows_t(device, S),
-                     _causal_row_np(S), heads={0, 13, H - 1})
+                     _causal_row_np(S), impl=impl, heads={0, 13, H - 1})
 
 
 @pytest.mark.parametrize("impl", ["hip", "hip_fused"])

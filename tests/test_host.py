@@ -36,7 +36,12 @@ def test_cpu_tensors_fail_loudly():
 def test_block_impl_and_bias_type_errors():
     q = torch.zeros(1, 64, 1, 64)
     with pytest.raises(ValueError):
-        ra.ring_attention(q, q, q, 2, block_impl="jax")  # ring.py:312 raises ValueError too
+        ra.ring_attention(q, q, q, 2, block_impl="triton")  # ring.py:312 raises ValueError too
+    # the reference's own two values are both accepted (ring.py:296-311): they get past the
+    # block_impl check and fail on the CPU tensors like any other call
+    for impl in ("jax", "pallas", "hip", "hip_fused"):
+        with pytest.raises(RuntimeError, match="no CPU fallback"):
+            ra.ring_attention(q, q, q, 2, block_impl=impl)
     with pytest.raises(TypeError):
         ra.ring_attention(q, q, q, 2, bias_fn="causal")  # neither a BiasFn nor a callable
     with pytest.raises(TypeError):
@@ -165,3 +170,67 @@ def test_shard_view_is_zero_copy():
     s = rr._shard_bhld(x, 1, 4)
     assert s.shape == (2, 3, 4, 4) and s.data_ptr() == x[:, 4:].data_ptr()
     assert torch.equal(s[1, 2, 3], x[1, 7, 2])
+
+
+def test_launch_scheme_per_block_impl():
+    q = torch.zeros(1, 64, 1, 64, dtype=torch.bfloat16)
+    plain = rr._RingPlan(q, q, 4, ra.causal_bias(), None, None)
+    dense = rr._RingPlan(q, q, 4, lambda q_ids, kv_ids: torch.zeros(1, 1, 16, 16),
+                         {"q_ids": torch.zeros(1, 64)}, {"kv_ids": torch.zeros(1, 64)})
+    # the reference's default spelling picks the scheme; its "jax" is the plain per-step loop
+    assert rr._launch_whole_ring("pallas", plain) and not rr._launch_whole_ring("pallas", dense)
+    assert not rr._launch_whole_ring("jax", plain) and not rr._launch_whole_ring("hip", plain)
+    assert rr._launch_whole_ring("hip_fused", plain) and rr._launch_whole_ring("hip_fused", dense)
+    import inspect
+    for f in (ra.ring_attention, ra.ring_self_attention, ra.ring_attention_with_lse):
+        assert inspect.signature(f).parameters["block_impl"].default == "pallas"  # ring.py:255
+
+
+def test_plans_are_cached_per_bias_arrays():
+    ra.clear_plan_cache()
+    q = torch.zeros(2, 64, 2, 64, dtype=torch.bfloat16)
+    seg = torch.arange(64)[None].repeat(2, 1) // 10
+    fn = ra.causal_bias() + ra.segment_bias()
+    a = rr._plan_for(q, q, 4, fn, {"q_segment_ids": seg}, {"kv_segment_ids": seg})
+    assert rr._plan_for(q, q, 4, fn, {"q_segment_ids": seg}, {"kv_segment_ids": seg}) is a
+    assert rr._plan_for(q, q, 4, ra.causal_bias() + ra.segment_bias(), {"q_segment_ids": seg},
+                        {"kv_segment_ids": seg}) is a           # an equal description, not the same object
+    assert rr._plan_for(q, q, 2, fn, {"q_segment_ids": seg}, {"kv_segment_ids": seg}) is not a
+    seg2 = seg.clone()
+    assert rr._plan_for(q, q, 4, fn, {"q_segment_ids": seg2}, {"kv_segment_ids": seg2}) is not a
+    seg += 1                                                    # in place: a new version of the same tensor
+    b = rr._plan_for(q, q, 4, fn, {"q_segment_ids": seg}, {"kv_segment_ids": seg})
+    assert b is not a and torch.equal(b.q_seg, seg.to(torch.int32))
+    # positions are read back on the host when a plan is made: the offsets follow the array
+    pos = torch.arange(64)[None].repeat(2, 1)
+    p1 = rr._plan_for(q, q, 4, ra.causal_bias(), {"q_positions": pos}, {})
+    pos += 5
+    p2 = rr._plan_for(q, q, 4, ra.causal_bias(), {"q_positions": pos}, {})
+    assert p1.q_off == [0, 16, 32, 48] and p2.q_off == [5, 21, 37, 53]
+    for i in range(20):                                         # bounded
+        rr._plan_for(q, q, 4, ra.sliding_window_bias(i + 1), None, None)
+    assert len(rr._PLAN_CACHE) <= rr._PLAN_CACHE_SIZE
+    ra.clear_plan_cache()
+    assert not rr._PLAN_CACHE
+
+
+def test_a_callable_bias_is_built_in_bounded_chunks():
+    q = torch.zeros(1, 256, 1, 64, dtype=torch.bfloat16)
+    calls = []
+
+    def fn(q_ids, kv_ids):
+        calls.append((int(q_ids[0, 0]), int(kv_ids[0, 0])))
+        return torch.zeros(1, 1, q_ids.shape[1], kv_ids.shape[1])
+
+    ids = torch.arange(256)[None]
+    plan = rr._RingPlan(q, q, 32, fn, {"q_ids": ids}, {"kv_ids": ids})
+    chunks = list(rr._row_chunks(plan, 3))
+    assert [len(c) for c in chunks] == [16, 16]                 # what one launch walks
+    assert [s for c in chunks for s, _ in c] == [(3 - t) % 32 for t in range(32)]   # ring order, ring.py:51-55
+    assert len(calls) == 32 and all(a == 24 for a, _ in calls)  # one block per pair, each built once
+    old = rr._DENSE_BLOCKS_BYTES
+    try:
+        rr._DENSE_BLOCKS_BYTES = 3 * 8 * 8 * 4                  # three 8 x 8 blocks
+        assert [len(c) for c in rr._row_chunks(plan, 0)] == [3] * 10 + [2]
+    finally:
+        rr._DENSE_BLOCKS_BYTES = old
