@@ -23,8 +23,19 @@
  *  - carries and accumulators are fp32 and contiguous: o/dq/dk/dv [B, H, L, D],
  *    m/l/lse/delta [B, H, L];
  *  - prefix masks are read as booleans: any non-zero value marks a prefix token;
- *  - D must be 64 or 128 and equal for q, k and v (the reference's kernels assume
- *    dk == dv too, ring_kernel.py:170,175); lengths may be any positive number.
+ *  - D must be 64 or 128 and equal for q, k and v; lengths may be any positive number.
+ *
+ * Limits against the reference's call surface (RA_ERR_HEAD_DIM / RA_ERR_SHAPE / RA_ERR_BIAS):
+ *  - one head dim for q, k and v: dk != dv is not supported.  The reference's fused kernels assume
+ *    dk == dv as well (ring_kernel.py:170,175 index o with dim_k); only its "jax" block functions
+ *    (ring.py:58-76,140-157) take a different dv.
+ *  - D in {64, 128} at this boundary; a host pads smaller head dims with zero columns (exact: zero
+ *    columns add nothing to a dot product).  Head dims above 128 are not supported.
+ *  - operands are bf16 (fp32 accumulation, fp32 carries, statistics and accumulators): a host
+ *    holding fp32 or fp16 arrays rounds them on entry.  The reference computes in the dtype of
+ *    its inputs (fp32 in its tests, ring_test.py:70-72).
+ *  - token positions (q_offset / kv_offset + index) lie in [0, RA_MAX_POSITION); shards hold at
+ *    most 2^24 tokens, RA_MAX_SEGMENT_SHARD under a segment bias.
  */
 #ifndef RING_ATTENTION_HIP_H
 #define RING_ATTENTION_HIP_H
@@ -59,6 +70,9 @@ extern "C" {
  * is walked as several shorter ones: the block step is associative over key/value shards and
  * independent over query rows (ring.py:58-76). */
 #define RA_MAX_SEGMENT_SHARD 65536
+/* Token positions (offset + index) must stay below this; RA_ERR_BIAS beyond.  A window wider than
+ * any position difference (>= 2^30) masks nothing and is treated as 2^30. */
+#define RA_MAX_POSITION ((1 << 30) - (1 << 16))
 
 #define RA_DTYPE_BF16 0
 #define RA_DTYPE_F32 1

@@ -36,7 +36,10 @@ int check_tensor(const char* name, const ra_tensor& t) {
   return RA_OK;
 }
 
-constexpr int64_t kMaxPos = (int64_t)1 << 30;
+// Token positions (offset + index) stay below 2^30 - 2^16 and the window is clamped to 2^30: every
+// position difference, with a window and a tile added, then fits 32 bits in the kernels.
+constexpr int64_t kMaxPos = ((int64_t)1 << 30) - (1 << 16);
+constexpr int kMaxWindow = 1 << 30;  // wider than any position difference: masks nothing more
 constexpr int kMaxLen = 1 << 24;
 constexpr int kMaxSegLen = 65536;  // tile-list capacity of the kernels (1024 tiles x 64)
 
@@ -79,8 +82,8 @@ int check_bias(const ra_bias& b, int Lq, int Lk) {
       return fail(RA_ERR_BIAS, "dense bias strides: stride_q must be at least Lk, stride_b / stride_h "
                                "non-negative (0 broadcasts)");
   }
-  if (b.q_offset < 0 || b.kv_offset < 0 || b.q_offset > kMaxPos || b.kv_offset > kMaxPos)
-    return fail(RA_ERR_BIAS, "token offsets must lie in [0, 2^30]");
+  if (b.q_offset < 0 || b.kv_offset < 0 || b.q_offset + Lq > kMaxPos || b.kv_offset + Lk > kMaxPos)
+    return fail(RA_ERR_BIAS, "token positions (offset + index) must lie in [0, 2^30 - 2^16)");
   return RA_OK;
 }
 
@@ -91,7 +94,7 @@ ra::TensorArg to_arg(const ra_tensor& t) {
 ra::BiasArgs to_bias(const ra_bias& b) {
   ra::BiasArgs r;
   r.flags = b.flags;
-  r.window = b.window;
+  r.window = b.window < kMaxWindow ? b.window : kMaxWindow;
   r.q_off = (int)b.q_offset;
   r.kv_off = (int)b.kv_offset;
   r.q_seg = b.q_segment_ids;

@@ -176,14 +176,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(av), "v"(bv));
   };
   if (GENERAL && tid < 64) {
-    // row l32 of the 32 x 16 operand is [i, i, 1, 1, 0 ...] with i = l32 the query's index in the
+    // row l32 of the 32 x 16 operand is [i, i, 1, 1, 1, 0 ...] with i = l32 the query's index in the
     // tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
     bf16x8 rf;
 #pragma unroll
     for (int e = 0; e < 8; ++e) rf[e] = (bf16_t)0.f;
     if (g == 0) {
       rf[0] = rf[1] = (bf16_t)(float)l32;
-      rf[2] = rf[3] = (bf16_t)1.0f;
+      rf[2] = rf[3] = rf[4] = (bf16_t)1.0f;
     }
     s_ramp[tid] = rf;
   }
@@ -402,10 +402,14 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       }
     }
   };
-  // converts the awaited tile's per-row word and publishes it (the caller has waited for it)
-  auto store_stat = [&](int buf) {
+  // The awaited tile's per-row word (the caller has waited for its load) is fetched, converted and
+  // published.  In two steps where operand fetches are in flight: LDS answers a wave in order, so
+  // using the word right behind its fetch would wait for every fetch issued before it.
+  auto fetch_stat = [&](int buf) -> unsigned {
     asm volatile("" ::: "memory");  // the read below stays behind the wait for the load
-    const unsigned x = s_raw[buf][tid];
+    return s_raw[buf][tid];
+  };
+  auto publish_stat = [&](unsigned x, int buf) {
     // lse -> -lse * log2(e), but -inf for a fully masked row (lse = -inf) so that its P is 0;
     // delta -> -delta, but 0 for the NaN that a fully masked output row produces
     float v = __uint_as_float(x) * st_mul;
@@ -414,6 +418,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     if (GENERAL) o = st_class >= 2 ? x : o;
     *(unsigned*)(&s_stat[0][0] + buf * STAT_BYTES + st_dst) = o;
   };
+  auto store_stat = [&](int buf) { publish_stat(fetch_stat(buf), buf); };
 
   // per-lane LDS offsets of the operand fetches (the tile buffer and the 16-row step fold into
   // the instructions' immediate offsets)
@@ -512,6 +517,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     tb.dense_mul = kLog2e * inv_res;
     tb.dense = nullptr;
     tb.dense_vs = 1;
+    tb.dense_vec = 0;
     tb.var_limit = a.Lq - (qt0 + 4 * g);
     const int rel0 = (q_off + qt0 + 4 * g) - (kv_off + kw + l32);
     const int* ids = (const int*)(stat_rd + ids_buf * STAT_BYTES);
@@ -679,10 +685,18 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   const char* st_run = st_src;
   const unsigned q_dst0 = RA_LDS_ADDR(&s_q[0][0]) + wave_u * 8 * ROWB;
   const unsigned do_dst0 = RA_LDS_ADDR(&s_do[0][0]) + wave_u * 8 * ROWB;
+  // The first PFT operand fragments of an iteration's dV / dK products, fetched in the tail of the
+  // iteration before (the tile they come from has been visible for two barriers by then): the
+  // fetch pipeline does not start from empty behind every barrier.
+  bf16x8 frc[PFT];
   auto seek_plain = [&](int tile) {
     q_run = qbase + (long long)(tile * kQTile + 8 * wave_u) * a.q.sl;
     do_run = dobase + (long long)(tile * kQTile + 8 * wave_u) * a.dout.sl;
     st_run = st_src + 4ll * (tile * kQTile + st_row);
+    // a stretch begins with phase 0: its first products take tile i - 1 from buffer NB - 1
+#pragma unroll
+    for (int op = 0; op < PFT; ++op)
+      frc[op] = tr_frag((op & 1) ? s_q[NB - 1] : s_do[NB - 1], op / (2 * DB), (op >> 1) % DB);
   };
 
   // The same iteration for a stretch of plain tiles: tiles i-1, i and i+1 are plain and tile i+3
@@ -711,10 +725,11 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     const char* dop = s_do[PHP];
     const char* qn = s_q[PH1];
     const char* don = s_do[PH1];
-    // operands of the dV / dK products come from tile i-1, visible since two barriers ago
+    // operands of the dV / dK products come from tile i-1, visible since two barriers ago; the
+    // first PFT of them were requested by the previous iteration (or by seek_plain)
     bf16x8 frb[4 * DB];
 #pragma unroll
-    for (int op = 0; op < PFT; ++op) frb[op] = tr_frag((op & 1) ? qp : dop, op / (2 * DB), (op >> 1) % DB);
+    for (int op = 0; op < PFT; ++op) frb[op] = frc[op];
     // all but the loads of tile i+2 have landed: this wave's share of tile i+1 is in LDS.  The
     // barrier is issued without a fence: the only LDS operations in flight are the PFT operand
     // fetches above, and what other waves need (the statistics stored half an iteration ago) is
@@ -773,26 +788,33 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       __builtin_amdgcn_sched_barrier(0);
     }
     // S(i+1), dP(i+1) with P(i), dS(i) in their shadow: one score element per MFMA, the chain of
-    // an element (exp2, product, packing) spread over consecutive slots
+    // an element (exp2, product, packing) spread over consecutive slots.  (Spreading the chain over
+    // the dV / dK slots as well - they carry two operand fetches each but no arithmetic - made the
+    // kernel 2 % slower: those slots are bound by their fetches, and vector instructions between
+    // them delay the fetches.)
     float pe[16], de[16];
     constexpr int EPO = 16 / (2 * KS) > 0 ? 16 / (2 * KS) : 1;
+    unsigned raw_word = 0;
     if (GENERAL && alibi_on) {
       // ALiBi of tile i+1 through the matrix unit: the score accumulators receive
-      //   [r, r, 1, 1] x [s_hi, s_lo, c_hi, c_lo] = s r + c = -slope |q_pos - kv_pos| (score units)
+      //   [r, r, 1, 1, 1] x [s_hi, s_lo, c_hi, c_mid, c_lo] = s r + c = -slope |q_pos - kv_pos| (score units)
       // with s = +-slope (the sign of the stretch), r the query's index in the tile and
-      // c = s (position of the tile's first query - kv_pos), both split into two bf16 words, so
-      // that the chain below needs no instruction for the bias.  Where the bias is large the
-      // split's error (2^-17 relative) is too, but there the probability is nil.
+      // c = s (position of the tile's first query - kv_pos); s is split into two bf16 words
+      // and c into three (c grows with the distance between the shards: three words carry it to
+      // fp32 accuracy, what an addition in the score chain would give), so that the chain below
+      // needs no instruction for the bias.
       const int rel_t = q_off + (tile_base + i + 1) * kQTile - (kv_off + kw + l32);
       const float ali_c = ali_s * (float)rel_t;
       const bf16_t c_hi = (bf16_t)ali_c;
-      const bf16_t c_lo = (bf16_t)(ali_c - (float)c_hi);
+      const bf16_t c_mid = (bf16_t)(ali_c - (float)c_hi);
+      const bf16_t c_lo = (bf16_t)((ali_c - (float)c_hi) - (float)c_mid);
       bf16x8 bq;
       bq[0] = ali_s_hi;
       bq[1] = ali_s_lo;
       bq[2] = c_hi;
-      bq[3] = c_lo;
-      bq[4] = bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
+      bq[3] = c_mid;
+      bq[4] = c_lo;
+      bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
       mfma_scores_v(SN, s_ramp[lane], bq);
     }
 #pragma unroll
@@ -803,7 +825,13 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       if (op == 2) {
         // the per-row word of tile i+2 is the oldest load but those of its tile and of tile i+3
         RA_WAIT_VMCNT(2 * LPT - 1);
-        store_stat(PH2);
+        raw_word = fetch_stat(PH2);
+      }
+      if (op == 2 + PFN) publish_stat(raw_word, PH2);  // behind as many fetches as are kept in flight
+      // the next iteration's first dV / dK operands: tile i, which it finds in buffer PH
+      if (op >= 2 * KS - PFT) {
+        const int o2 = op - (2 * KS - PFT);
+        frc[o2] = tr_frag((o2 & 1) ? s_q[PH] : s_do[PH], o2 / (2 * DB), (o2 >> 1) % DB);
       }
 #pragma unroll
       for (int e = 0; e < EPO; ++e) {
@@ -1085,14 +1113,14 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     }
     if (GENERAL) s_q1[tid] = qf[1];
     if (GENERAL && tid < 64) {
-      // row l32 of the 32 x 16 operand is [j, j, 1, 1, 0 ...] with j = l32 the key's index in the
+      // row l32 of the 32 x 16 operand is [j, j, 1, 1, 1, 0 ...] with j = l32 the key's index in the
       // tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
       bf16x8 rf;
 #pragma unroll
       for (int e = 0; e < 8; ++e) rf[e] = (bf16_t)0.f;
       if (g == 0) {
         rf[0] = rf[1] = (bf16_t)(float)l32;
-        rf[2] = rf[3] = (bf16_t)1.0f;
+        rf[2] = rf[3] = rf[4] = (bf16_t)1.0f;
       }
       s_ramp[tid] = rf;
     }
@@ -1397,6 +1425,11 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     tb.dense_mul = kLog2e / a.scale_res;
     tb.dense = nullptr;
     tb.dense_vs = 1;
+    tb.dense_vec = 0;
+    if (DENSE) {
+      const float* head = dense_ptr + b * bs.dense_sb + h * bs.dense_sh;
+      tb.dense_vec = kt0 + kDqKeyTile <= a.Lk && ((((uintptr_t)head) | ((uintptr_t)bs.dense_sq << 2)) & 15) == 0;
+    }
     const int var0 = kt0 + 4 * g;
     tb.var_limit = a.Lk - var0;
     const int rel0 = (q_off + qi) - (kv_off + var0);
@@ -1610,9 +1643,12 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 #pragma unroll
     for (int op = 0; op < PF; ++op) frb[op] = tr_frag(kp, op / DB, op % DB);
     if (!late_half) {
-      // all loads but the two of tile i+2 have landed: this wave's share of tile i+1 is in LDS
+      // all loads but the two of tile i+2 have landed: this wave's share of tile i+1 is in LDS.
+      // The barrier is issued without a fence: a stretch writes nothing to LDS but through the
+      // tile loads, which the counter above covers, and the operand fetches just issued (two LDS
+      // instructions each) may stay in flight across it instead of being drained.
       __builtin_amdgcn_s_waitcnt(0x0f72);
-      __syncthreads();
+      asm volatile("s_waitcnt lgkmcnt(%0)\n\ts_barrier" : : "n"(2 * PF) : "memory");
     }
     bf16x8 dsf[2];
     dsf[0] = __builtin_bit_cast(bf16x8, dsw[0]);
@@ -1683,23 +1719,26 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     };
     if (GENERAL && alibi_on) {
       // ALiBi of tile i+1 through the matrix unit: the accumulators start from
-      //   [j, j, 1, 1] x [s_hi, s_lo, c_hi, c_lo] = s j + c = -slope |q_pos - kv_pos| (score units)
+      //   [j, j, 1, 1, 1] x [s_hi, s_lo, c_hi, c_mid, c_lo] = s j + c = -slope |q_pos - kv_pos| (score units)
       // with s = +-slope (the sign of the stretch), j the key's index in the tile and
-      // c = -s (q_pos - position of the tile's first key), both split into two bf16 words, so
-      // that the chain below needs no instruction for the bias.  Where the bias is large the
-      // split's error (2^-17 relative) is too, but there the probability is nil.
+      // c = -s (q_pos - position of the tile's first key); s is split into two bf16 words and c
+      // into three (c grows with the distance between the shards: three words carry it to fp32
+      // accuracy, what an addition in the score chain would give), so that the chain below needs
+      // no instruction for the bias.
       // (recomputed per tile from the lane number: the loop has no register to carry it in)
       const int ramp_lane = tid & 63;
       const int rel_i = q_off + q_first + (tid >> 6) * 32 + (ramp_lane & 31) - (kv_off + (run_tile0 + i + 1) * kDqKeyTile);
       const float ali_c = -ali_s * (float)rel_i;
       const bf16_t c_hi = (bf16_t)ali_c;
-      const bf16_t c_lo = (bf16_t)(ali_c - (float)c_hi);
+      const bf16_t c_mid = (bf16_t)(ali_c - (float)c_hi);
+      const bf16_t c_lo = (bf16_t)((ali_c - (float)c_hi) - (float)c_mid);
       bf16x8 bq;
       bq[0] = ali_s_hi;
       bq[1] = ali_s_lo;
       bq[2] = c_hi;
-      bq[3] = c_lo;
-      bq[4] = bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
+      bq[3] = c_mid;
+      bq[4] = c_lo;
+      bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
       f32x16 z;
 #pragma unroll
       for (int r = 0; r < 16; ++r) z[r] = 0.f;

@@ -204,6 +204,7 @@ struct TileBias {
   int var_limit; // varying-side indices >= var_limit (relative to var0) are out of range
   const float* dense;   // dense bias element of (fixed index, var0); natural-log units
   long long dense_vs;   // its stride along the varying side (1 when the keys vary)
+  int dense_vec;        // keys vary, the whole block is in range and rows are 16-byte aligned: vector loads
 };
 
 // Branch-free per element: the uniform `flags` only shape a handful of per-lane constants up
@@ -223,18 +224,23 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
   if (!TERMS) flags &= RA_BIAS_CAUSAL | RA_BIAS_WINDOW;
   const bool causal = flags & RA_BIAS_CAUSAL, window = flags & RA_BIAS_WINDOW;
   const bool segment = flags & RA_BIAS_SEGMENT, prefix = flags & RA_BIAS_PREFIX;
+  const bool dense_vec = DENSE && __builtin_amdgcn_readfirstlane(tb.dense_vec) != 0;
   int lo = 0, hi = tb.var_limit - 1;  // off >= var_limit: out of range
   int pre_lo = -kFar, pre_hi = kFar;  // outside [pre_lo, pre_hi]: rel < 0, masked unless both sides are prefix
+  // |rel0| < 2^30 and window <= 2^30 (the host checks positions and clamps the window), so the sums
+  // below stay inside 32 bits; the prefix interval is 2^29 wide on its open side, and a block
+  // further than that from the diagonal is clamped to "every rel < 0" / "every rel >= 0"
+  const int relp = max(min(rel0, kFar - 64), 64 - kFar);
   if (QFIXED) {  // rel = rel0 - off: rel < 0 <=> off > rel0, rel >= w <=> off <= rel0 - w, -rel >= w <=> off >= rel0 + w
     if (causal) hi = min(hi, rel0);
     if (window) lo = max(lo, rel0 - tb.window + 1);
     if (window && !causal) hi = min(hi, rel0 + tb.window - 1);
-    if (prefix) pre_hi = rel0;
+    if (prefix) pre_hi = relp;
   } else {  // rel = rel0 + off: rel < 0 <=> off < -rel0, rel >= w <=> off >= w - rel0, -rel >= w <=> off <= -rel0 - w
     if (causal) lo = max(lo, -rel0);
     if (window) hi = min(hi, tb.window - 1 - rel0);
     if (window && !causal) lo = max(lo, 1 - rel0 - tb.window);
-    if (prefix) pre_lo = -rel0;
+    if (prefix) pre_lo = -relp;
   }
   // off in [lo, hi] <=> (unsigned)(off - lo) <= (unsigned)(hi - lo); an empty interval (hi < lo)
   // becomes lo = 1 << 30, span = 0: no off in 0..63 passes
@@ -256,9 +262,16 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
       if (PRE) vp = *(const i32x4*)(var_pre + 8 * bb);
       float dn[4] = {0.f, 0.f, 0.f, 0.f};
       if (DENSE) {
+        if (QFIXED && dense_vec) {
+          // a lane's four keys are 16 contiguous bytes of its row: one load instead of four
+          const f32x4 v4 = *(const f32x4*)(tb.dense + 8 * bb);
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (8 * bb + c < tb.var_limit) dn[c] = QFIXED ? tb.dense[8 * bb + c] : tb.dense[(8 * bb + c) * tb.dense_vs];
+          for (int c = 0; c < 4; ++c) dn[c] = v4[c];
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; ++c)
+            if (8 * bb + c < tb.var_limit) dn[c] = QFIXED ? tb.dense[8 * bb + c] : tb.dense[(8 * bb + c) * tb.dense_vs];
+        }
       }
 #pragma unroll
       for (int c = 0; c < 4; ++c) {

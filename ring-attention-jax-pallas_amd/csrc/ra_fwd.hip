@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (GENERAL) s_q1[tid] = qf[1];
     if (PARK2) s_q2[tid] = qf[2];
     if (GENERAL && tid < 64) {
-      // row (32 kb + l32) of the 32 x 16 operand is [j, j, 1, 1, 0 ...] with j the key's index in
+      // row (32 kb + l32) of the 32 x 16 operand is [j, j, 1, 1, 1, 0 ...] with j the key's index in
       // the tile (exact in bf16); lanes 32..63 hold the other eight columns, all zero
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         for (int e = 0; e < 8; ++e) rf[e] = (bf16_t)0.f;
         if (g == 0) {
           rf[0] = rf[1] = (bf16_t)(float)(32 * kb + l32);
-          rf[2] = rf[3] = (bf16_t)1.0f;
+          rf[2] = rf[3] = rf[4] = (bf16_t)1.0f;
         }
         if (!PARK2) s_ramp[64 * kb + tid] = rf;
         else if (tid < 32) s_ramp[32 * kb + tid] = rf;
@@ -529,6 +529,11 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     tb.dense_mul = kLog2e * inv_scale2;
     tb.dense = nullptr;
     tb.dense_vs = 1;
+    tb.dense_vec = 0;
+    if (DENSE) {
+      const float* head = dense_ptr + b * bs.dense_sb + h * bs.dense_sh;
+      tb.dense_vec = kt0 + kKeyTile <= a.Lk && ((((uintptr_t)head) | ((uintptr_t)bs.dense_sq << 2)) & 15) == 0;
+    }
     float mx = RA_NEG_INF;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
@@ -915,23 +920,26 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       bf16x8 fr[NOPA];
       if (GENERAL && alibi_on) {
         // ALiBi of tile i+1 through the matrix unit: the accumulators start from
-        //   [j, j, 1, 1] x [s_hi, s_lo, c_hi, c_lo] = s j + c = -slope |q_pos - kv_pos| / scale2
+        //   [j, j, 1, 1, 1] x [s_hi, s_lo, c_hi, c_mid, c_lo] = s j + c = -slope |q_pos - kv_pos| / scale2
         // with s = +-slope / scale2 (the sign of the stretch), j the key's index in the tile and
-        // c = -s (q_pos - position of the tile's first key), both split into two bf16 words, so
-        // that the score chain below needs no instruction for the bias.  Where the bias is
-        // large the split's error (2^-17 relative) is too, but there the probability is nil.
+        // c = -s (q_pos - position of the tile's first key); s is split into two bf16 words and c
+        // into three (c grows with the distance between the shards: three words carry it to fp32
+        // accuracy, what an addition in the score chain would give), so that the score chain
+        // below needs no instruction for the bias.
         // (recomputed per tile from the lane number: the loop has no register to carry it in)
         const int ramp_lane = tid & 63;
         const int rel_i = q_off + q0 + (tid >> 6) * 32 + (ramp_lane & 31) - (kv_off + (tile_base + i + 1) * kKeyTile);
         const float ali_c = -ali_s * (float)rel_i;
         const bf16_t c_hi = (bf16_t)ali_c;
-        const bf16_t c_lo = (bf16_t)(ali_c - (float)c_hi);
+        const bf16_t c_mid = (bf16_t)(ali_c - (float)c_hi);
+        const bf16_t c_lo = (bf16_t)((ali_c - (float)c_hi) - (float)c_mid);
         bf16x8 bq;
         bq[0] = ali_s_hi;
         bq[1] = ali_s_lo;
         bq[2] = c_hi;
-        bq[3] = c_lo;
-        bq[4] = bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
+        bq[3] = c_mid;
+        bq[4] = c_lo;
+        bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
         f32x16 z;
 #pragma unroll
         for (int r = 0; r < 16; ++r) z[r] = 0.f;

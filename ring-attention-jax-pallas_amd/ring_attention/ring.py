@@ -394,8 +394,8 @@ class _RingPlan:
         expect = (starts[:, :, None] + torch.arange(L, device=pos.device)[None, None, :]).reshape(self.B, S)
         if not torch.equal(expect, pos) or not bool((starts == starts[:1]).all()):
             return None
-        if int(starts.min()) < 0 or int(starts.max()) + L > (1 << 30):
-            return None  # outside the offset range of the C ABI
+        if int(starts.min()) < 0 or int(starts.max()) + L > _lib.RA_MAX_POSITION:
+            return None  # outside the position range of the C ABI
         return [int(x) for x in starts[0].tolist()]
 
     def live_steps(self, qs: Optional[int], ks: Optional[int]) -> int:
@@ -499,9 +499,9 @@ def _ring_forward(q, k, v, plan: _RingPlan, sm_scale, out_dtype, carries_out=Non
         qr = _shard_bhld(q, r, Lq)
         for t in range(n):
             src = (r - t) % n  # ring.py:51-55: after t rotations device r holds shard r - t
+            bias = plan.block_bias(r, src)  # ring.py:107 (a callable's dense block is built here)
             with timer.span("fwd", r, src):
-                fwd_block(qr, _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk),
-                          plan.block_bias(r, src), o, m, l, sm_scale)
+                fwd_block(qr, _shard_bhld(k, src, Lk), _shard_bhld(v, src, Lk), bias, o, m, l, sm_scale)
             if carries_out is not None:
                 carries_out.append((r, t, o.clone(), m.clone(), l.clone()))
         finalize_carry(o, m, l, _shard_bhld(out, r, Lq), lse[r])

@@ -84,6 +84,11 @@ def test_check_accepts_good_params(lib):
     (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_DENSE), setattr(p.bias, "dense_bias", 0x3002),
                 setattr(p.bias, "dense_stride_q", 64)), -4),
     (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL), setattr(p.bias, "q_offset", -5)), -5),
+    # positions (offset + index) stay below RA_MAX_POSITION: the last token of the shard counts
+    (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL),
+                setattr(p.bias, "q_offset", _lib.RA_MAX_POSITION - p.Lq + 1)), -5),
+    (lambda p: (setattr(p.bias, "flags", _lib.RA_BIAS_CAUSAL),
+                setattr(p.bias, "kv_offset", _lib.RA_MAX_POSITION - p.Lk + 1)), -5),
 ])
 def test_fwd_step_rejects_bad_params_without_a_gpu(lib, mutate, code):
     p = _good_fwd()
@@ -91,6 +96,23 @@ def test_fwd_step_rejects_bad_params_without_a_gpu(lib, mutate, code):
     assert lib.ra_fwd_step_check(C.byref(p)) == code
     assert lib.ra_fwd_step(C.byref(p), None) == code  # validation comes before any HIP call
     assert lib.ra_last_error() != b""
+
+
+def test_position_and_window_limits(lib):
+    # the largest positions and any window width pass the checks (a window wider than every
+    # position difference masks nothing and is clamped inside the library)
+    p = _good_fwd()
+    p.bias.flags = _lib.RA_BIAS_CAUSAL | _lib.RA_BIAS_WINDOW
+    p.bias.window = 2 ** 31 - 1
+    p.bias.q_offset = _lib.RA_MAX_POSITION - p.Lq
+    p.bias.kv_offset = _lib.RA_MAX_POSITION - p.Lk
+    assert lib.ra_fwd_step_check(C.byref(p)) == 0
+    # a step against keys 2^30 positions behind a window of 2^31 - 1 still has work; one beyond a
+    # small window has none
+    p.bias.kv_offset = 0
+    assert lib.ra_step_is_skippable(C.byref(p.bias), p.Lq, p.Lk) == 0
+    p.bias.window = 1000
+    assert lib.ra_step_is_skippable(C.byref(p.bias), p.Lq, p.Lk) == 1
 
 
 def test_bwd_step_rejects_bad_params_without_a_gpu(lib):

@@ -370,6 +370,82 @@ def test_block_api_matches_reference_contract(device):
         assert mx <= GRAD_TOL and fro <= GRAD_TOL
 
 
+def _block_step_against_oracle(device, fn, ofn, q_off, kv_off, Lq, Lk, D, qkw=None, kvkw=None, seed=3, check_m=True):
+    """One block step (fwd_block, then bwd_block on its own normalised output) at the given shard
+    positions against the oracle's block functions fed the dense bias of explicit positions."""
+    B, H = 1, 2
+    q, k, v, do = R.make_inputs(seed, B, Lq, Lk, H, D)
+    hq, hk, hv, hdo = (np.ascontiguousarray(np.transpose(x, (0, 2, 1, 3))) for x in (q, k, v, do))
+    tq, tk, tv, tdo = (_dev(x, device, torch.bfloat16) for x in (hq, hk, hv, hdo))
+    qpos = np.broadcast_to(q_off + np.arange(Lq, dtype=np.int64), (B, Lq))
+    kpos = np.broadcast_to(kv_off + np.arange(Lk, dtype=np.int64), (B, Lk))
+    dense = ofn(**dict(qkw or {}, q_positions=qpos), **dict(kvkw or {}, kv_positions=kpos))  # [b, h | 1, lq, lk]
+    dense = np.broadcast_to(dense, (B, H, Lq, Lk)).astype(np.float64)
+    if fn.alibi_slopes is not None:
+        fn = ra.BiasFn(fn.causal, fn.window, fn.segments, fn.prefix, fn.alibi_slopes.to(device))
+    bb = ra.BlockBias(fn, q_off, kv_off, *(None if x is None else _dev(x, device) for x in (
+        (qkw or {}).get("q_segment_ids"), (kvkw or {}).get("kv_segment_ids"),
+        (qkw or {}).get("q_prefix_mask"), (kvkw or {}).get("kv_prefix_mask"))))
+    scale = 1 / math.sqrt(D)
+    o, m, l = rr.init_carry(B, H, Lq, D, device)
+    o, m, l = ra.fwd_block(tq, tk, tv, bb, o, m, l, scale)
+    wo, wm, wl = R.fwd_block(hq.astype(np.float64), hk.astype(np.float64), hv.astype(np.float64), dense,
+                             np.zeros((B, H, Lq, D)), np.full((B, H, Lq), -np.inf), np.zeros((B, H, Lq)), scale)
+    live = np.isfinite(wm)
+    assert live.any()
+    np.testing.assert_array_equal(np.isneginf(m.cpu().numpy()), ~live)
+    got_out = (o / l[..., None]).cpu().numpy()[live]
+    got_lse = (m + torch.log(l)).cpu().numpy()[live]
+    want_out, want_lse = (wo / wl[..., None])[live], (wm + np.log(wl))[live]
+    e_out, e_lse = np.abs(got_out - want_out).max(), np.abs(got_lse - want_lse).max()
+    # |lse| grows with the bias: hold it to the fp32 resolution of its own size on top of the bound
+    assert e_out <= OUT_TOL and e_lse <= LSE_TOL + 4e-7 * np.abs(want_lse).max(), (e_out, e_lse)
+    if check_m:
+        assert np.abs(m.cpu().numpy()[live] - wm[live]).max() <= 1e-4 + 4e-7 * np.abs(wm[live]).max()
+    out = torch.nan_to_num(o / l[..., None])
+    L = m + torch.log(l)
+    dq, dk, dv = ra.bwd_block(tq, tk, tv, bb, out, L, tdo, scale)
+    w_out = np.where(live[..., None], wo / np.where(wl == 0, 1, wl)[..., None], 0.0)
+    w_do = np.where(live[..., None], hdo.astype(np.float64), 0.0)       # dead rows contribute nothing
+    w_L = np.where(live, wm + np.log(np.where(wl == 0, 1, wl)), 0.0)
+    w_dense = np.where(live[..., None], dense, 0.0)
+    wdq, wdk, wdv = R.bwd_block(hq.astype(np.float64), hk.astype(np.float64), hv.astype(np.float64), w_dense,
+                                w_out, w_L, w_do, scale)
+    for nm, got, ref in (("dq", dq.cpu().numpy()[live], wdq[live]), ("dk", dk.cpu().numpy(), wdk),
+                         ("dv", dv.cpu().numpy(), wdv)):
+        mx, fro = _rel(got, ref)
+        assert mx <= GRAD_TOL and fro <= GRAD_TOL, (nm, mx, fro)
+    return e_out, e_lse
+
+
+@pytest.mark.parametrize("q_off,kv_off", [(0, rr._lib.RA_MAX_POSITION - 384), (rr._lib.RA_MAX_POSITION - 256, 0),
+                                          (1000, 1000 + (1 << 29) + 5), (0, 64)])
+def test_prefix_block_step_far_from_the_diagonal(device, q_off, kv_off):
+    """A lone block step whose key/value shard lies up to 2^30 positions before or behind the query
+    shard (the widest the C ABI takes): behind it only prefix & prefix pairs are unmasked, before
+    it every pair is."""
+    Lq, Lk = 256, 384
+    rng = np.random.default_rng(1)
+    qpm = (rng.random((1, Lq)) < 0.5).astype(np.int32)
+    kpm = (rng.random((1, Lk)) < 0.5).astype(np.int32)
+    _block_step_against_oracle(device, ra.prefix_lm_bias(), R.make_bias_fn(use_prefix=True), q_off, kv_off, Lq, Lk, 64,
+                               {"q_prefix_mask": qpm}, {"kv_prefix_mask": kpm})
+
+
+@pytest.mark.parametrize("q_off,kv_off,causal", [(100000, 0, True), (0, 300000, False), (5000, 4000, False),
+                                                 (200000, 0, True)])
+def test_alibi_block_step_far_from_the_diagonal(device, q_off, kv_off, causal):
+    """ALiBi on a lone block step far from the diagonal: slope x distance reaches 6000 - 19000 (the
+    largest slope is 1/16 here), and the weights inside the block must still follow the bias of
+    the oracle - the kernels add the term through the matrix unit, the distance-dependent constant
+    split into three bf16 words.  (Beyond a few hundred thousand positions fp32 itself - the
+    reference's bias dtype - no longer resolves the bias to 1e-3.)"""
+    H = 2
+    sl = R.alibi_slopes(H)
+    fn = ra.alibi_bias(sl) + (ra.causal_bias() if causal else ra.BiasFn())
+    _block_step_against_oracle(device, fn, R.make_bias_fn(causal=causal, alibi=sl), q_off, kv_off, 1024, 1024, 128)
+
+
 # ---- arbitrary bias_fn callables: the dense additive block of ring.py:107 ---------------------------
 def _callable_check(device, name, B, Sq, Sk, H, D, n, torch_fn, numpy_fn, qkw, kvkw, seed=0):
     """ring_attention with a Python callable as bias_fn against the dense closed form with the

@@ -166,4 +166,4 @@ def test_unrounded_fp32_inputs_against_the_reference_tolerance(device, name, see
           f"worst excess {np.max(err - (1e-3 + 1e-2 * np.abs(want))):.2e}", flush=True)
     assert err.max() <= OUT_TOL
     assert err.max() <= floor.max() + 5e-3                   # the kernels add little to the rounding of the inputs
-    assert inside.mean() >= 0.9
+    assert inside.mean() >= 0.97                             # measured: 97.9 % (96 elements) .. 100 %
