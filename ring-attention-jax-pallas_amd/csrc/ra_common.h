@@ -217,7 +217,7 @@ struct TileBias {
 template <bool QFIXED, bool DENSE, bool TERMS>
 RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, int fixed_pre,
                        const int* var_seg, const int* var_pre) {
-  constexpr int kFar = 1 << 29;
+  constexpr int kFar = 1 << 30;
   // one value per wave (a block belongs to one wave's rows and one tile): say so, or the compiler
   // carries every flag test as a lane mask
   int flags = __builtin_amdgcn_readfirstlane(tb.flags);
@@ -228,25 +228,24 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
   int lo = 0, hi = tb.var_limit - 1;  // off >= var_limit: out of range
   int pre_lo = -kFar, pre_hi = kFar;  // outside [pre_lo, pre_hi]: rel < 0, masked unless both sides are prefix
   // |rel0| < 2^30 and window <= 2^30 (the host checks positions and clamps the window), so the sums
-  // below stay inside 32 bits; the prefix interval is 2^29 wide on its open side, and a block
-  // further than that from the diagonal is clamped to "every rel < 0" / "every rel >= 0"
-  const int relp = max(min(rel0, kFar - 64), 64 - kFar);
+  // below stay inside 32 bits, and the prefix interval - open to 2^30 on one side - holds every
+  // rel0 without a clamp (an instruction more per block costs the 256-register kernels a spill)
   if (QFIXED) {  // rel = rel0 - off: rel < 0 <=> off > rel0, rel >= w <=> off <= rel0 - w, -rel >= w <=> off >= rel0 + w
     if (causal) hi = min(hi, rel0);
     if (window) lo = max(lo, rel0 - tb.window + 1);
     if (window && !causal) hi = min(hi, rel0 + tb.window - 1);
-    if (prefix) pre_hi = relp;
+    if (prefix) pre_hi = rel0;
   } else {  // rel = rel0 + off: rel < 0 <=> off < -rel0, rel >= w <=> off >= w - rel0, -rel >= w <=> off <= -rel0 - w
     if (causal) lo = max(lo, -rel0);
     if (window) hi = min(hi, tb.window - 1 - rel0);
     if (window && !causal) lo = max(lo, 1 - rel0 - tb.window);
-    if (prefix) pre_lo = -relp;
+    if (prefix) pre_lo = -rel0;
   }
   // off in [lo, hi] <=> (unsigned)(off - lo) <= (unsigned)(hi - lo); an empty interval (hi < lo)
   // becomes lo = 1 << 30, span = 0: no off in 0..63 passes
   const bool none = hi < lo;
   const unsigned nlo = (unsigned)(none ? -(1 << 30) : -lo), span = (unsigned)(none ? 0 : hi - lo);
-  const unsigned pnlo = (unsigned)(-pre_lo), pspan = (unsigned)(pre_hi - pre_lo);
+  const unsigned pnlo = (unsigned)(-pre_lo), pspan = (unsigned)pre_hi - (unsigned)pre_lo;  // < 2^31 under a prefix term
   const int seg_ref = fixed_seg;
   const int pre_on = (prefix && fixed_pre != 0) ? -1 : 0;  // all ones where this lane's side carries the flag
   const float slope = -tb.slope2;

@@ -5,7 +5,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libringattn_hip.so")
+# the library built in-tree; RING_ATTENTION_HIP_LIB names another build of the same ABI
+LIB_PATH = os.environ.get("RING_ATTENTION_HIP_LIB") or os.path.join(_HERE, "libringattn_hip.so")
 
 RA_BIAS_CAUSAL = 1
 RA_BIAS_WINDOW = 2
