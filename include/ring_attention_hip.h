@@ -36,6 +36,8 @@
  *    its inputs (fp32 in its tests, ring_test.py:70-72).
  *  - token positions (q_offset / kv_offset + index) lie in [0, RA_MAX_POSITION); shards hold at
  *    most 2^24 tokens, RA_MAX_SEGMENT_SHARD under a segment bias.
+ *  - row strides (ra_tensor.stride_l) lie in [D, 2^27] elements: rows do not overlap, and the
+ *    rows one wavefront moves stay within a 32-bit byte offset of each other.
  */
 #ifndef RING_ATTENTION_HIP_H
 #define RING_ATTENTION_HIP_H
@@ -77,7 +79,8 @@ extern "C" {
 #define RA_DTYPE_BF16 0
 #define RA_DTYPE_F32 1
 
-/* bf16 tensor view [B, H, L, D] with explicit element strides (D contiguous). */
+/* bf16 tensor view [B, H, L, D] with explicit element strides (D contiguous; strides multiples of 8,
+ * D <= stride_l <= 2^27). */
 typedef struct ra_tensor {
   const void* ptr;
   int64_t stride_b;

@@ -28,11 +28,18 @@ int hip_fail(hipError_t e, const char* what) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int check_tensor(const char* name, const ra_tensor& t) {
+// The kernels reach the rows that one wave moves (up to 16 of them) through an unsigned 32-bit byte
+// offset per lane from the wave's first row: rows may not overlap and the row stride stays below 2^27.
+constexpr int64_t kMaxRowStride = (int64_t)1 << 27;
+
+int check_tensor(const char* name, const ra_tensor& t, int D) {
   if (!t.ptr) return fail(RA_ERR_NULL, "%s.ptr is NULL", name);
   if (!aligned16(t.ptr)) return fail(RA_ERR_ALIGN, "%s.ptr is not 16-byte aligned", name);
   if ((t.stride_b % 8) || (t.stride_h % 8) || (t.stride_l % 8))
     return fail(RA_ERR_ALIGN, "%s strides must be multiples of 8 elements (16 bytes)", name);
+  if (t.stride_l < D || t.stride_l > kMaxRowStride)
+    return fail(RA_ERR_SHAPE, "%s.stride_l = %lld: the row stride must lie in [D, 2^27] elements", name,
+                (long long)t.stride_l);
   return RA_OK;
 }
 
@@ -543,9 +550,9 @@ int ra_fwd_step_check(const ra_fwd_step_params* p) {
   if (!p) return fail(RA_ERR_NULL, "params is NULL");
   int rc = check_dims(p->B, p->H, p->Lq, p->Lk, p->D);
   if (rc) return rc;
-  if ((rc = check_tensor("q", p->q))) return rc;
-  if ((rc = check_tensor("k", p->k))) return rc;
-  if ((rc = check_tensor("v", p->v))) return rc;
+  if ((rc = check_tensor("q", p->q, p->D))) return rc;
+  if ((rc = check_tensor("k", p->k, p->D))) return rc;
+  if ((rc = check_tensor("v", p->v, p->D))) return rc;
   if (!p->o || !p->m || !p->l) return fail(RA_ERR_NULL, "carry pointer (o, m or l) is NULL");
   if (!aligned16(p->o)) return fail(RA_ERR_ALIGN, "o is not 16-byte aligned");
   if (!(p->sm_scale > 0.f) || p->sm_scale > 3.0e38f)
@@ -557,10 +564,10 @@ int ra_bwd_step_check(const ra_bwd_step_params* p) {
   if (!p) return fail(RA_ERR_NULL, "params is NULL");
   int rc = check_dims(p->B, p->H, p->Lq, p->Lk, p->D);
   if (rc) return rc;
-  if ((rc = check_tensor("q", p->q))) return rc;
-  if ((rc = check_tensor("k", p->k))) return rc;
-  if ((rc = check_tensor("v", p->v))) return rc;
-  if ((rc = check_tensor("dout", p->dout))) return rc;
+  if ((rc = check_tensor("q", p->q, p->D))) return rc;
+  if ((rc = check_tensor("k", p->k, p->D))) return rc;
+  if ((rc = check_tensor("v", p->v, p->D))) return rc;
+  if ((rc = check_tensor("dout", p->dout, p->D))) return rc;
   if (!p->lse || !p->delta) return fail(RA_ERR_NULL, "lse or delta is NULL");
   if (!p->dq || !p->dk || !p->dv) return fail(RA_ERR_NULL, "gradient accumulator (dq, dk or dv) is NULL");
   if (!aligned16(p->dq) || !aligned16(p->dk) || !aligned16(p->dv))
@@ -649,7 +656,7 @@ int ra_bwd_delta_passes(const void* out, int32_t out_dtype, int64_t out_stride_p
   int rc = check_dims(B, H, Lq, 1, D);
   if (rc) return rc;
   if ((int64_t)n_passes * B * H > (1 << 20)) return fail(RA_ERR_SHAPE, "n_passes*B*H too large");
-  if ((rc = check_tensor("dout", *dout))) return rc;
+  if ((rc = check_tensor("dout", *dout, D))) return rc;
   if (out_dtype != RA_DTYPE_BF16 && out_dtype != RA_DTYPE_F32)
     return fail(RA_ERR_DTYPE, "unknown out_dtype %d", out_dtype);
   if (!aligned16(out) || (out_stride_pass % 8) || (out_stride_b % 8) || (out_stride_h % 8) || (out_stride_l % 8) ||

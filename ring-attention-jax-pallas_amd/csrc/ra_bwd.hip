@@ -346,15 +346,17 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   constexpr int NLD = 8 / RPI;
   constexpr int LPT = 2 * NLD + 1;  // vector-memory instructions per wave and tile
   int ld_row[NLD], ld_off[NLD];
-  unsigned q_voff[NLD], do_voff[NLD];  // per-lane byte offsets inside a group of RPI rows
+  // per-lane byte offsets from the wave's first row; the second group of RPI rows (D = 128) rides
+  // on the same scalar base through its distance, less the 1 KiB instruction offset of the paired load
+  unsigned q_voff[NLD], do_voff[NLD];
 #pragma unroll
   for (int t = 0; t < NLD; ++t) {
     const int rrow = 8 * wave + RPI * t + lane / CPR;
     const int pc = lane % CPR;
     ld_row[t] = rrow;
     ld_off[t] = ((tile_off<D>(rrow, pc) - rrow * ROWB) >> 4) * 8;
-    q_voff[t] = (unsigned)(((long long)(lane / CPR) * a.q.sl + ld_off[t]) * 2);
-    do_voff[t] = (unsigned)(((long long)(lane / CPR) * a.dout.sl + ld_off[t]) * 2);
+    q_voff[t] = (unsigned)(((long long)(lane / CPR + RPI * t) * a.q.sl + ld_off[t]) * 2 - 1024 * t);
+    do_voff[t] = (unsigned)(((long long)(lane / CPR + RPI * t) * a.dout.sl + ld_off[t]) * 2 - 1024 * t);
   }
   // The per-row words of a tile: lane l of every wave fetches word class (l / 8) % NSTAT of row
   // 8 * wave + l % 8 (lanes 32..63 repeat lanes 0..31) straight into LDS, like the tile itself and
@@ -387,8 +389,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       const bf16_t* qs = qbase + (long long)(q0 + 8 * wave_u) * a.q.sl;
       const bf16_t* ds = dobase + (long long)(q0 + 8 * wave_u) * a.dout.sl;
       if (NLD == 2) {
-        global_to_lds16_s_x2(qs, q_voff[0], qs + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1], q_dst);
-        global_to_lds16_s_x2(ds, do_voff[0], ds + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1], do_dst);
+        global_to_lds16_s_x2(qs, q_voff[0], q_voff[NLD - 1], q_dst);
+        global_to_lds16_s_x2(ds, do_voff[0], do_voff[NLD - 1], do_dst);
       } else {
         global_to_lds16_s(qs, q_voff[0], q_dst);
         global_to_lds16_s(ds, do_voff[0], do_dst);
@@ -764,12 +766,12 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
         st_run += kQTile * 4;
       }
       if (op == 1) {
-        if (NLD == 2) global_to_lds16_s_x2(q_run, q_voff[0], q_run + (long long)RPI * a.q.sl - 512, q_voff[NLD - 1], q_dst0 + PH3 * TILE_BYTES);
+        if (NLD == 2) global_to_lds16_s_x2(q_run, q_voff[0], q_voff[NLD - 1], q_dst0 + PH3 * TILE_BYTES);
         else global_to_lds16_s(q_run, q_voff[0], q_dst0 + PH3 * TILE_BYTES);
         q_run += (long long)kQTile * a.q.sl;
       }
       if (op == 2) {
-        if (NLD == 2) global_to_lds16_s_x2(do_run, do_voff[0], do_run + (long long)RPI * a.dout.sl - 512, do_voff[NLD - 1], do_dst0 + PH3 * TILE_BYTES);
+        if (NLD == 2) global_to_lds16_s_x2(do_run, do_voff[0], do_voff[NLD - 1], do_dst0 + PH3 * TILE_BYTES);
         else global_to_lds16_s(do_run, do_voff[0], do_dst0 + PH3 * TILE_BYTES);
         do_run += (long long)kQTile * a.dout.sl;
       }

@@ -168,10 +168,13 @@ RA_DEV void global_to_lds16(const void* gptr, unsigned lds_addr) {
 RA_DEV void global_to_lds16_s(const void* sbase, unsigned voff, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %0" : : "s"(sbase), "v"(voff), "s"(lds_addr) : "memory", "m0");
 }
-RA_DEV void global_to_lds16_s_x2(const void* sbase0, unsigned voff0, const void* sbase1_minus_1k, unsigned voff1,
-                                 unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %4\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %0\n\tglobal_load_lds_dwordx4 %3, %2 offset:1024"
-               : : "s"(sbase0), "v"(voff0), "s"(sbase1_minus_1k), "v"(voff1), "s"(lds_addr) : "memory", "m0");
+// Both pieces go through ONE scalar base: the second piece's distance from the first, minus the
+// 1 KiB of the instruction offset, travels in its per-lane offset (an unsigned 32-bit byte count,
+// which bounds the row stride at the ABI).  A second base would cost two scalar additions per call,
+// and the loops that call this are bound by instruction issue.
+RA_DEV void global_to_lds16_s_x2(const void* sbase, unsigned voff0, unsigned voff1_minus_1k, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %0\n\tglobal_load_lds_dwordx4 %2, %0 offset:1024"
+               : : "s"(sbase), "v"(voff0), "v"(voff1_minus_1k), "s"(lds_addr) : "memory", "m0");
 }
 // one dword per lane: lane l's word lands at lds_addr + 4 l
 RA_DEV void global_to_lds4(const void* gptr, unsigned lds_addr) {

@@ -301,14 +301,15 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const int rrow = 8 * wave + RPI * t + lane / CPR;
     const int pc = lane % CPR;
     const int lc = (tile_off<D>(rrow, pc) - rrow * (D * 2)) >> 4;  // logical chunk stored at pc
-    k_voff[t] = (unsigned)(((long long)(lane / CPR) * a.k.sl + lc * 8) * 2);
-    v_voff[t] = (unsigned)(((long long)(lane / CPR) * a.v.sl + lc * 8) * 2);
+    // from the wave's first row: the second group of RPI rows (D = 128) rides on the same scalar base
+    k_voff[t] = (unsigned)(((long long)(lane / CPR + RPI * t) * a.k.sl + lc * 8) * 2);
+    v_voff[t] = (unsigned)(((long long)(lane / CPR + RPI * t) * a.v.sl + lc * 8) * 2);
   }
   auto issue_rows = [&](const bf16_t* base, const unsigned (&voff)[NLD], long long sl, int k0, unsigned dst) {
     if (k0 + kKeyTile <= a.Lk) {
       const bf16_t* sb = base + (long long)(k0 + 8 * wave_u) * sl;  // wave-uniform: scalar registers
-      if (NLD == 2) global_to_lds16_s_x2(sb, voff[0], sb + (long long)RPI * sl - 512, voff[NLD - 1], dst);
-      else global_to_lds16_s(sb, voff[0], dst);
+      global_to_lds16_s(sb, voff[0], dst);
+      if (NLD == 2) global_to_lds16_s(sb, voff[NLD - 1], dst + RPI * (D * 2));
     } else {  // last, partial tile: rows past the end repeat the last row (masked later)
 #pragma unroll
       for (int t = 0; t < NLD; ++t) {
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // the issuing waves
   auto issue_part = [&](const bf16_t* base, const unsigned (&voff)[NLD], long long sl, int k0, unsigned dst, int t) {
     if (k0 + kKeyTile <= a.Lk) {
-      global_to_lds16_s(base + (long long)(k0 + 8 * wave_u + RPI * t) * sl, voff[t], dst + RPI * t * (D * 2));
+      global_to_lds16_s(base + (long long)(k0 + 8 * wave_u) * sl, voff[t], dst + RPI * t * (D * 2));
     } else {
       const int gr = min(k0 + ld_row(t), a.Lk - 1);
       global_to_lds16(base + (long long)gr * sl + ld_koff(t), dst + RPI * t * (D * 2));
@@ -817,7 +818,6 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // are complete: straight-line code, no classification, no flags, scalar running addresses.
   const bf16_t* k_run = kbase;
   const bf16_t* v_run = vbase;
-  const long long k_part = (long long)RPI * a.k.sl, v_part = (long long)RPI * a.v.sl;
   const unsigned k_dst0 = RA_LDS_ADDR(&s_k[0][0]) + wave_u * 8 * (D * 2);
   const unsigned v_dst0 = RA_LDS_ADDR(&s_v[0][0]) + wave_u * 8 * (D * 2);
   auto seek_plain = [&](int ordinal) {  // the iteration with this ordinal is the next to run
@@ -970,7 +970,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         SN[op & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[op], op < 2 ? q0 : (op < 4 ? q1 : (op < 6 ? q2 : qf[op >> 1])), SN[op & 1], 0, 0, 0);
         if (op == NOPA / 4) global_to_lds16_s(k_run, k_voff[0], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES);
         if (NLD == 2 && op == NOPA * 3 / 4)
-          global_to_lds16_s(k_run + k_part, k_voff[NLD - 1], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES + RPI * (D * 2));
+          global_to_lds16_s(k_run, k_voff[NLD - 1], k_dst0 + ((PAR + 3) & 3) * TILE_BYTES + RPI * (D * 2));
         links_of_slot(op);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -990,7 +990,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         oacc[op % DB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
             fr[op], __builtin_bit_cast(bf16x8, pw[op / DB]), oacc[op % DB], 0, 0, 0);
         if (op == NOPB / 4) global_to_lds16_s(v_run, v_voff[0], v_dst);
-        if (NLD == 2 && op == NOPB * 3 / 4) global_to_lds16_s(v_run + v_part, v_voff[NLD - 1], v_dst + RPI * (D * 2));
+        if (NLD == 2 && op == NOPB * 3 / 4) global_to_lds16_s(v_run, v_voff[NLD - 1], v_dst + RPI * (D * 2));
         links_of_slot(NOPA + op);
 #pragma unroll
         for (int x = 0; x < maxima_in(op); ++x) {
