@@ -36,7 +36,7 @@
  *    its inputs (fp32 in its tests, ring_test.py:70-72).
  *  - token positions (q_offset / kv_offset + index) lie in [0, RA_MAX_POSITION); shards hold at
  *    most 2^24 tokens, RA_MAX_SEGMENT_SHARD under a segment bias.
- *  - row strides (ra_tensor.stride_l) lie in [D, 2^27] elements: rows do not overlap, and the
+ *  - row strides (ra_tensor.stride_l) lie in [D, RA_MAX_ROW_STRIDE] elements: rows do not overlap, and the
  *    rows one wavefront moves stay within a 32-bit byte offset of each other.
  */
 #ifndef RING_ATTENTION_HIP_H
@@ -75,6 +75,8 @@ extern "C" {
 /* Token positions (offset + index) must stay below this; RA_ERR_BIAS beyond.  A window wider than
  * any position difference (>= 2^30) masks nothing and is treated as 2^30. */
 #define RA_MAX_POSITION ((1 << 30) - (1 << 16))
+/* ra_tensor.stride_l lies in [D, RA_MAX_ROW_STRIDE] elements; RA_ERR_SHAPE beyond. */
+#define RA_MAX_ROW_STRIDE (1 << 27)
 
 #define RA_DTYPE_BF16 0
 #define RA_DTYPE_F32 1

@@ -30,7 +30,7 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) ==
 
 // The kernels reach the rows that one wave moves (up to 16 of them) through an unsigned 32-bit byte
 // offset per lane from the wave's first row: rows may not overlap and the row stride stays below 2^27.
-constexpr int64_t kMaxRowStride = (int64_t)1 << 27;
+constexpr int64_t kMaxRowStride = RA_MAX_ROW_STRIDE;
 
 int check_tensor(const char* name, const ra_tensor& t, int D) {
   if (!t.ptr) return fail(RA_ERR_NULL, "%s.ptr is NULL", name);

@@ -822,6 +822,9 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
       if (op + PFN < 2 * KS) fra[op + PFN] = nat_frag(((op + PFN) & 1) ? don : qn, (op + PFN) >> 1);
+      // one s_waitcnt for the operands of two MFMAs: the compiler waits in front of whatever reads a
+      // fetched register, and a wait costs this wave an issue slot like any instruction
+      if (!(op & 1)) asm volatile("" : : "v"(fra[op]), "v"(fra[op + 1]));
       if (op & 1) mfma_scores(PN, fra[op], vfa[op >> 1]);
       else mfma_scores(SN, fra[op], kfa[op >> 1]);
       if (op == 2) {

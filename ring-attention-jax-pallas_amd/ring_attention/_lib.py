@@ -18,6 +18,7 @@ RA_DTYPE_BF16 = 0
 RA_ERR_TOO_LARGE = -8  # a whole-ring launch cannot hold the passes: use the split entry points
 RA_MAX_SEGMENT_SHARD = 65536  # longest shard that one call takes under a segment bias
 RA_MAX_POSITION = (1 << 30) - (1 << 16)  # token positions (offset + index) stay below this
+RA_MAX_ROW_STRIDE = 1 << 27  # elements between two rows of a q / k / v / dO view, at most
 RA_DTYPE_F32 = 1
 
 

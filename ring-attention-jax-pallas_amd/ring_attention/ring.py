@@ -112,10 +112,12 @@ def _view_bhld(t: torch.Tensor) -> _lib.RaTensor:
 
 
 def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
-    """bf16, unit inner stride, 16-byte aligned rows."""
+    """[b, l, h, d] as the kernels take it: bf16, unit inner stride, 16-byte aligned rows that do not
+    overlap and lie within the row stride the C ABI admits; anything else is copied."""
     if t.dtype != torch.bfloat16:
         t = t.to(torch.bfloat16)
-    ok = t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+    ok = (t.stride(-1) == 1 and all(s % 8 == 0 for s in t.stride()[:-1]) and t.data_ptr() % 16 == 0
+          and t.shape[-1] <= t.stride(1) <= _lib.RA_MAX_ROW_STRIDE)
     return t if ok else t.contiguous()
 
 

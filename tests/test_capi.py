@@ -118,7 +118,7 @@ def test_position_and_window_limits(lib):
 def test_row_stride_limits(lib):
     # rows may not overlap (stride_l >= D) and the row stride stays within 2^27 elements: the kernels
     # reach the rows one wavefront moves through a 32-bit byte offset from the wavefront's first row
-    for bad in (0, -128, 64, 2 ** 27 + 8):
+    for bad in (0, -128, 64, _lib.RA_MAX_ROW_STRIDE + 8):
         p = _good_fwd()
         p.k.stride_l = bad
         assert p.D == 128 and lib.ra_fwd_step_check(C.byref(p)) == -2, bad
@@ -126,7 +126,7 @@ def test_row_stride_limits(lib):
         p = _good_bwd()
         p.dout.stride_l = min(bad, 56)  # D = 64 there
         assert lib.ra_bwd_step_check(C.byref(p)) == -2, bad
-    for good in (128, 136, 2 ** 27):
+    for good in (128, 136, _lib.RA_MAX_ROW_STRIDE):
         p = _good_fwd()
         p.v.stride_l = good
         assert lib.ra_fwd_step_check(C.byref(p)) == 0, good

@@ -167,3 +167,33 @@ def test_unrounded_fp32_inputs_against_the_reference_tolerance(device, name, see
     assert err.max() <= OUT_TOL
     assert err.max() <= floor.max() + 5e-3                   # the kernels add little to the rounding of the inputs
     assert inside.mean() >= 0.97                             # measured: 97.9 % (96 elements) .. 100 %
+
+
+@pytest.mark.parametrize("row_stride,S,n", [(2 * 128 + 8, 1024, 2), (1 << 22, 512, 2), (1 << 27, 64, 1)])
+def test_row_strides_up_to_the_limit(device, row_stride, S, n):
+    """q, k, v and dO as views with a padded, a wide and the widest row stride the C ABI admits (2^27
+    elements: the rows one wavefront moves then lie up to 1.9 GB apart, reached through a 32-bit
+    byte offset per lane).  The storage is allocated, never filled: only the 256-byte rows are
+    touched.  Same bits as the contiguous tensors, whatever the addresses."""
+    B, H, D = 1, 2, 128
+    print(f"[strides] row stride {row_stride} elements, S={S}, ring={n}", flush=True)
+    q, k, v, do = R.make_inputs(31, B, S, S, H, D)
+
+    def strided(x, dt):
+        t = torch.empty_strided((B, S, H, D), (S * row_stride, row_stride, D, 1), dtype=dt, device=device)
+        t.copy_(_dev(x, device, dt))
+        return t
+
+    def run(make, impl):
+        tq, tk, tv = (make(x, torch.bfloat16).requires_grad_(True) for x in (q, k, v))
+        out, lse = ra.ring_attention_with_lse(tq, tk, tv, n, bias_fn=ra.causal_bias(), out_dtype=torch.float32,
+                                              block_impl=impl)
+        out.backward(make(do, torch.float32))
+        torch.cuda.synchronize()
+        return [out.detach().cpu(), lse.cpu()] + [t.grad.float().cpu() for t in (tq, tk, tv)]
+
+    for impl in IMPLS:
+        want = run(lambda x, dt: _dev(x, device, dt), impl)
+        got = run(strided, impl)
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), impl

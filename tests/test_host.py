@@ -234,3 +234,19 @@ def test_a_callable_bias_is_built_in_bounded_chunks():
         assert [len(c) for c in rr._row_chunks(plan, 0)] == [3] * 10 + [2]
     finally:
         rr._DENSE_BLOCKS_BYTES = old
+
+
+def test_views_the_kernels_cannot_take_are_copied():
+    # a view is passed through when its rows are 16-byte aligned, do not overlap and lie within the
+    # row stride of the C ABI; otherwise the host makes a contiguous copy
+    base = torch.zeros((2, 16, 4, 64 + 8), dtype=torch.bfloat16)
+    padded = base[..., :64]                       # row stride 4 * 72, inner stride 1
+    assert rr._kernel_ready(padded) is padded
+    odd = torch.zeros((2, 16, 4, 65), dtype=torch.bfloat16)[..., :64]   # strides not multiples of 8
+    assert rr._kernel_ready(odd).is_contiguous()
+    same_row = torch.zeros((2, 1, 4, 64), dtype=torch.bfloat16).expand(2, 16, 4, 64)   # row stride 0
+    got = rr._kernel_ready(same_row)
+    assert got.is_contiguous() and got.shape == same_row.shape
+    heads_interleaved = torch.zeros((2, 4, 16, 64), dtype=torch.bfloat16).permute(0, 2, 1, 3)  # [b, l, h, d] view, row stride 64
+    assert rr._kernel_ready(heads_interleaved) is heads_interleaved
+    assert rr._kernel_ready(torch.zeros((1, 8, 1, 64))).dtype == torch.bfloat16
