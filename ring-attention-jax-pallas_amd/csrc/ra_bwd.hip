@@ -819,14 +819,17 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
       bq[5] = bq[6] = bq[7] = (bf16_t)0.f;
       mfma_scores_v(SN, s_ramp[lane], bq);
     }
+    fra[PFN] = nat_frag((PFN & 1) ? don : qn, PFN >> 1);
 #pragma unroll
     for (int op = 0; op < 2 * KS; ++op) {
-      if (op + PFN < 2 * KS) fra[op + PFN] = nat_frag(((op + PFN) & 1) ? don : qn, (op + PFN) >> 1);
-      // one s_waitcnt for the operands of two MFMAs: the compiler waits in front of whatever reads a
-      // fetched register, and a wait costs this wave an issue slot like any instruction
-      if (!(op & 1)) asm volatile("" : : "v"(fra[op]), "v"(fra[op + 1]));
       if (op & 1) mfma_scores(PN, fra[op], vfa[op >> 1]);
       else mfma_scores(SN, fra[op], kfa[op >> 1]);
+      // The wait for the next MFMA's operand goes right behind this MFMA, in front of the slot's operand
+      // fetch and vector work (the compiler waits in front of whatever reads a fetched register): a
+      // lone wave issues MFMA, s_waitcnt, ds_read, 4 vector instructions in 36 cycles, and the same
+      // instructions with the wait behind them, in front of the next MFMA, in 40 to 48.
+      if (op + 1 < 2 * KS) asm volatile("" : : "v"(fra[op + 1]));
+      if (op + 1 + PFN < 2 * KS) fra[op + 1 + PFN] = nat_frag(((op + 1 + PFN) & 1) ? don : qn, (op + 1 + PFN) >> 1);
       if (op == 2) {
         // the per-row word of tile i+2 is the oldest load but those of its tile and of tile i+3
         RA_WAIT_VMCNT(2 * LPT - 1);
@@ -1678,7 +1681,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       // its dQ^T block while the other runs its S^T / dP^T block.  Tiles i+2 and i+3 may still
       // be in flight (two loads each).
       __builtin_amdgcn_s_waitcnt(0x0f74);
-      __syncthreads();
+      barrier_bare();
 #pragma unroll
       for (int op = 0; op < PF; ++op) fra[op] = nat_frag((op & 1) ? vn : kn, op >> 1);
     }

@@ -176,6 +176,11 @@ RA_DEV void global_to_lds16_s_x2(const void* sbase, unsigned voff0, unsigned vof
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %0\n\tglobal_load_lds_dwordx4 %2, %0 offset:1024"
                : : "s"(sbase), "v"(voff0), "v"(voff1_minus_1k), "s"(lds_addr) : "memory", "m0");
 }
+// Workgroup barrier of the straight-line loops, whose only LDS writes are tile loads that the caller
+// counts with vmcnt: nothing is awaited, and LDS reads of this wave may stay in flight across it.
+// __syncthreads() puts a workgroup fence on either side of s_barrier, which costs the forward loop
+// 3 % and buys nothing there (in the generic iterations, which store to LDS, it costs nothing).
+RA_DEV void barrier_bare() { asm volatile("s_barrier" ::: "memory"); }
 // one dword per lane: lane l's word lands at lds_addr + 4 l
 RA_DEV void global_to_lds4(const void* gptr, unsigned lds_addr) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");

@@ -826,7 +826,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   };
   auto sync_plain = [&]() {
     __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));  // only the previous barrier's requests are in flight
-    __syncthreads();
+    barrier_bare();
   };
   const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
   // The key-side ids seen through the constant address space: with a wave-uniform index the
@@ -860,10 +860,10 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     const unsigned v_dst = v_dst0 + (late_half ? ((PAR + 3) & 3) : ((PAR + 2) & 3)) * TILE_BYTES;
     // ---- S(i+1) MFMAs, then O += P(i) V_i, with the softmax arithmetic of tile i and the row
     // maximum of S(i+1) in their shadow.  The chain of a pair of scores (scale and shift, exp2,
-    // pack, rounded row sum, exact row sum) is spread over five consecutive MFMA slots, one link
-    // per slot, so that no vector instruction waits for the result of the one before it and no
-    // slot carries both the exp2 pair of one chain and all three sum instructions of another
-    // (1.8 % of the kernel); the sixteen pairs of a lane
+    // pack, exact row sum) is spread over consecutive MFMA slots, one link per slot, so that no
+    // vector instruction waits for the result of the one before it and no slot carries both the
+    // exp2 pair of one chain and the sum instructions of another (1.8 % of the kernel); the
+    // rounded row sums wait for the end of their block (see links_of_slot); the sixteen pairs of a lane
     // are spread over both MFMA blocks so that every slot carries about the same vector work:
     // half of them (the first two operand fragments of P) in the score block, the other half in
     // the first three quarters of the output block, the row maxima in the slots that remain.
@@ -912,8 +912,21 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         if (slot_of(w) - 1 == gs) link1(w);
         if (slot_of(w) == gs) link2(w);
         if (slot_of(w) + 1 == gs) link3(w);
-        if (slot_of(w) + 2 == gs) link4(w);
         if (slot_of(w) + 3 == gs) link5(w);
+      }
+      // The rounded row sums go in two bursts, behind the last MFMA of either block: a dot-product
+      // instruction between two MFMAs holds up the matrix pipe (a hand-built copy of this loop runs
+      // at 53 cycles per MFMA with one v_dot2c per slot, at 42 with the same sixteen in two bursts,
+      // at 39 without them; a v_fma in its place costs a tenth of that).
+      if (gs == NOPA - 1) {
+#pragma unroll
+        for (int w = 0; w < 16; ++w)
+          if (slot_of(w) + 1 <= NOPA - 1) link4(w);
+      }
+      if (gs == NOPA + NOPB - 1) {
+#pragma unroll
+        for (int w = 0; w < 16; ++w)
+          if (slot_of(w) + 1 > NOPA - 1) link4(w);
       }
     };
     {
