@@ -208,6 +208,45 @@ def mfma_ceiling(torch, dev):
             "what": "v_mfma_f32_32x32x16_bf16 only, random operands in registers, one wave per SIMD, all CUs"}
 
 
+def coissue_probe(torch, dev):
+    """Table of the co-issue probe of libringattn_probe.so: shader-clock cycles per v_mfma_f32_32x32x16_bf16 and
+    SIMD when every MFMA of a loop is followed by a fixed group of other instructions, at one and at two waves
+    per SIMD (32 = the matrix pipe is busy all the time).  One workgroup per compute unit; a workgroup's time is that
+    of its slowest wave, the table holds the median over workgroups."""
+    import ctypes as C
+    from ring_attention import _lib
+    path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libringattn_probe.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: build the kernels first (__graft_entry__.build())")
+    lib = C.CDLL(path)
+    lib.ra_probe_coissue_cases.restype = C.c_int
+    lib.ra_probe_coissue_what.restype = C.c_char_p
+    lib.ra_probe_coissue_what.argtypes = [C.c_int]
+    lib.ra_probe_coissue.restype = C.c_int
+    lib.ra_probe_coissue.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    iters = 20000
+    cycles = torch.zeros(cus * 8, device=dev, dtype=torch.int64)
+    src = torch.zeros(cus * 16384, device=dev, dtype=torch.uint8)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    lines = [f"cycles of the shader clock per v_mfma_f32_32x32x16_bf16 and SIMD; loop of 8 MFMAs x {iters} trips, "
+             f"{cus} workgroups (slowest wave of each, median over workgroups)",
+             f"{'behind every MFMA':<84}{'1 wave/SIMD':>12}{'2 waves/SIMD':>13}"]
+    for c in range(lib.ra_probe_coissue_cases()):
+        row = []
+        for waves in (4, 8):
+            for n in (200, iters):  # a short launch first: code and clocks warm
+                rc = lib.ra_probe_coissue(cycles.data_ptr(), c, waves, cus, n, src.data_ptr(), stream)
+                if rc:
+                    raise RuntimeError(f"ra_probe_coissue failed with code {rc}")
+                torch.cuda.synchronize()
+            # the SIMD's older wave is served first and finishes early: a workgroup's time is its slowest wave's
+            med = cycles[:cus * waves].view(cus, waves).max(dim=1).values.float().median().item()
+            row.append(med / (iters * 8) / (waves // 4))
+        lines.append(f"{lib.ra_probe_coissue_what(c).decode():<84}{row[0]:>12.1f}{row[1]:>13.1f}")
+    return "\n".join(lines) + "\n"
+
+
 def cpu_baseline(D, config="sample"):
     """The numpy restatement of the reference algorithm (fp32, causal) timed on the host cores:
     a bounded sample with the workload's head dim (H=8, S=16384 as 4 shards of 4096), or
@@ -272,6 +311,9 @@ def main():
                          "under profiles/ and print it")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain elementwise copy of 1 GiB (calibrates HBM byte counters)")
+    ap.add_argument("--coissue-probe", action="store_true",
+                    help="no workload: print the table of what fits in the shadow of an MFMA (instruction groups "
+                         "behind every MFMA of a loop, cycles per MFMA) and exit")
     args = ap.parse_args()
     if args.pmc_summary:
         sys.stdout.write(pmc_summary(args.workload, *args.pmc_summary))
@@ -290,6 +332,9 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.coissue_probe:
+        sys.stdout.write(coissue_probe(torch, dev))
+        return
     w = WORKLOADS[args.workload]
     small = args.workload in ("C2", "C4", "C5", "CALLABLE")
     if args.steps is None:
