@@ -177,9 +177,8 @@ RA_DEV void global_to_lds16_s_x2(const void* sbase, unsigned voff0, unsigned vof
                : : "s"(sbase), "v"(voff0), "v"(voff1_minus_1k), "s"(lds_addr) : "memory", "m0");
 }
 // Workgroup barrier of the straight-line loops, whose only LDS writes are tile loads that the caller
-// counts with vmcnt: nothing is awaited, and LDS reads of this wave may stay in flight across it.
-// __syncthreads() puts a workgroup fence on either side of s_barrier, which costs the forward loop
-// 3 % and buys nothing there (in the generic iterations, which store to LDS, it costs nothing).
+// counts with vmcnt: nothing is awaited, and LDS reads of this wave may stay in flight across it
+// (__syncthreads() puts a workgroup fence on either side of s_barrier, which orders nothing there).
 RA_DEV void barrier_bare() { asm volatile("s_barrier" ::: "memory"); }
 // one dword per lane: lane l's word lands at lds_addr + 4 l
 RA_DEV void global_to_lds4(const void* gptr, unsigned lds_addr) {

@@ -839,7 +839,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   bf16_t ali_s_hi = (bf16_t)0.f, ali_s_lo = (bf16_t)0.f;
   auto plain_iteration = [&](auto parity, int i, f32x16 (&SC)[2], f32x16 (&SN)[2]) {
     constexpr int PAR = decltype(parity)::value;
-    constexpr int PF = TIGHT ? 2 : 3;  // these variants have four registers less to spare
+    constexpr int PF = TIGHT ? 2 : 4;  // operand fetches in flight; the TIGHT variants have no registers for more
     if (!late_half) sync_plain();
     const char* kt = s_k[(PAR + 1) & 3];
     const unsigned vt = PAR * TILE_BYTES;
@@ -915,9 +915,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         if (slot_of(w) + 3 == gs) link5(w);
       }
       // The rounded row sums go in two bursts, behind the last MFMA of either block: a dot-product
-      // instruction between two MFMAs holds up the matrix pipe (a hand-built copy of this loop runs
-      // at 53 cycles per MFMA with one v_dot2c per slot, at 42 with the same sixteen in two bursts,
-      // at 39 without them; a v_fma in its place costs a tenth of that).
+      // instruction between two MFMAs holds the matrix pipe up for 17-19 cycles, one of a burst for
+      // 5-9 (a v_fma_f32 in its place: 1).
       if (gs == NOPA - 1) {
 #pragma unroll
         for (int w = 0; w < 16; ++w)
