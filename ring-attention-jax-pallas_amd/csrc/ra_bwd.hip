@@ -1336,16 +1336,16 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
         global_to_lds16(vbase + (long long)gr * a.v.sl + ld_chunk, v_dst);
       }
     }
-    if (GENERAL && with_ids && tid < kDqKeyTile) {
-      int kk = min(k0 + tid, a.Lk - 1);
+    if (GENERAL && with_ids && lane < kDqKeyTile) {
+      int kk = min(k0 + lane, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
     }
   };
   auto store_ids = [&](int buf) {
-    if (GENERAL && tid < kDqKeyTile) {
-      s_seg[buf][tid] = seg_r;
-      s_pre[buf][tid] = pre_r;
+    if (GENERAL && lane < kDqKeyTile) {
+      s_seg[buf][lane] = seg_r;
+      s_pre[buf][lane] = pre_r;
     }
   };
 
@@ -1885,18 +1885,20 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
 #pragma unroll
       for (int r = 0; r < 16; ++r) s_a[r] = RA_NEG_INF;
     }
-    if (tid < kDqKeyTile) {
+    if (lane < kDqKeyTile) {
       // the stretch moved no ids: those of the two tiles in flight are fetched now (i is a
       // multiple of 6 here: tile i+1 lives in buffer 1, the ids of tile i+2 wait in registers
-      // for the top of the next iteration, as after a generic iteration)
+      // for the top of the next iteration, as after a generic iteration).  Every wave does this for
+      // itself, as it fetches and stores the ids in its generic iterations: the waves enter and
+      // leave their stretches at different tiles and must not depend on one another for the ids.
       int sbu;
       if (i + 1 < n) {
-        const int kk = min(tile_at(i + 1, sbu) * kDqKeyTile + tid, a.Lk - 1);
-        s_seg[1][tid] = kv_seg ? kv_seg[kk] : 0;
-        s_pre[1][tid] = kv_pre ? kv_pre[kk] : 0;
+        const int kk = min(tile_at(i + 1, sbu) * kDqKeyTile + lane, a.Lk - 1);
+        s_seg[1][lane] = kv_seg ? kv_seg[kk] : 0;
+        s_pre[1][lane] = kv_pre ? kv_pre[kk] : 0;
       }
       if (i + 2 < n) {
-        const int kk = min(tile_at(i + 2, sbu) * kDqKeyTile + tid, a.Lk - 1);
+        const int kk = min(tile_at(i + 2, sbu) * kDqKeyTile + lane, a.Lk - 1);
         if (kv_seg) seg_r = kv_seg[kk];
         if (kv_pre) pre_r = kv_pre[kk];
       }

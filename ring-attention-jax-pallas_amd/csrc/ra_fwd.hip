@@ -332,8 +332,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   auto issue_k = [&](int j, int buf) {
     const int k0 = j * kKeyTile;
     issue_rows(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + buf * TILE_BYTES + wave_u * 8 * (D * 2));
-    if (GENERAL && tid < kKeyTile) {
-      int kk = min(k0 + tid, a.Lk - 1);
+    if (GENERAL && lane < kKeyTile) {
+      int kk = min(k0 + lane, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
     }
@@ -355,18 +355,22 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     if (j < n && t < NLD) {
       const int k0 = tile_at(j, sb_unused) * kKeyTile;
       issue_part(kbase, k_voff, a.k.sl, k0, RA_LDS_ADDR(&s_k[0][0]) + (j & 3) * TILE_BYTES + wave_u * 8 * (D * 2), t);
-      if (GENERAL && !DEFER && t == 0 && tid < kKeyTile) {
-        int kk = min(k0 + tid, a.Lk - 1);
+      if (GENERAL && !DEFER && t == 0 && lane < kKeyTile) {
+        int kk = min(k0 + lane, a.Lk - 1);
         if (kv_seg) seg_r = kv_seg[kk];
         if (kv_pre) pre_r = kv_pre[kk];
       }
     }
   };
+  // The segment ids / prefix flags of a key tile.  EVERY wave fetches and stores them (the same
+  // values to the same LDS words): the waves of a workgroup enter and leave their straight-line
+  // stretches at different tiles (a window's lower edge, the diagonal), a stretch moves no ids,
+  // and a wave in a generic iteration must not depend on another wave being in one too.
   // the ids of K tile ordinal j, into registers (store_ids publishes them), where they do not
   // travel with the request
   auto fetch_ids = [&](int j) {
-    if (j < n && tid < kKeyTile) {
-      const int kk = min(tile_at(j, sb_unused) * kKeyTile + tid, a.Lk - 1);
+    if (j < n && lane < kKeyTile) {
+      const int kk = min(tile_at(j, sb_unused) * kKeyTile + lane, a.Lk - 1);
       if (kv_seg) seg_r = kv_seg[kk];
       if (kv_pre) pre_r = kv_pre[kk];
     }
@@ -378,9 +382,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     }
   };
   auto store_ids = [&](int buf) {
-    if (GENERAL && tid < kKeyTile) {
-      s_seg[buf][tid] = seg_r;
-      s_pre[buf][tid] = pre_r;
+    if (GENERAL && lane < kKeyTile) {
+      s_seg[buf][lane] = seg_r;
+      s_pre[buf][lane] = pre_r;
       seg_r = pre_r = 0;  // dead until the next request: not carried around the loops
     }
   };
@@ -1113,15 +1117,15 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
         for (int r = 0; r < 16; ++r) sa[0][r] = sa[1][r] = RA_NEG_INF;
       }
     }
-    // the plain iterations requested K tiles i .. i+2 without their ids: fetch them for the
-    // iterations that follow (the barrier at the top of iteration i publishes them)
-    if (GENERAL && tid < kKeyTile) {
+    // the plain iterations requested K tiles i .. i+2 without their ids: this wave fetches them
+    // for its own iterations that follow
+    if (GENERAL && lane < kKeyTile) {
 #pragma unroll
       for (int t = 0; t < 3; ++t) {
         if (i + t < n) {
-          const int kk = min(tile_at(i + t, sb_unused) * kKeyTile + tid, a.Lk - 1);
-          if (kv_seg) s_seg[(i + t) & 3][tid] = kv_seg[kk];
-          if (kv_pre) s_pre[(i + t) & 3][tid] = kv_pre[kk];
+          const int kk = min(tile_at(i + t, sb_unused) * kKeyTile + lane, a.Lk - 1);
+          if (kv_seg) s_seg[(i + t) & 3][lane] = kv_seg[kk];
+          if (kv_pre) s_pre[(i + t) & 3][lane] = kv_pre[kk];
         }
       }
     }

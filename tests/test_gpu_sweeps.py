@@ -93,7 +93,7 @@ def _against_dense_oracle(device, name, B, S, H, D, n, fn, ofn, qkw, kvkw, seed,
     return worst
 
 
-@pytest.mark.parametrize("seed", [0, 1])
+@pytest.mark.parametrize("seed", [0, 1, 2])
 def test_long_shard_configurations(device, seed):
     for case, kind, kw in _long_shard_cases(seed, 10):
         _against_dense_oracle(device, f"long shards {seed}.{case} {kind} D={kw['D']} n={kw['n']} S={kw['S']}", **kw)
@@ -197,3 +197,23 @@ def test_row_strides_up_to_the_limit(device, row_stride, S, n):
         got = run(strided, impl)
         for a, b in zip(got, want):
             assert torch.equal(a, b), impl
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_waves_enter_their_stretches_at_different_tiles_under_segments(device, D):
+    """A sliding window whose lower edge crosses a key/value shard: the later waves of a workgroup
+    lose keys to the window that its first wave still sees, so the waves enter their straight-line
+    stretches at different tiles.  Under a segment bias a wave in a generic iteration needs the
+    key ids of its tile, and a stretch moves none: every wave fetches them for itself (when only
+    the first wave did, the others read whatever the compute unit's LDS held from the launch
+    before - the ids of another document, now and then).  Several calls in a row: the stale
+    contents were those of the previous step kernel."""
+    B, S, H, n, window = 1, 5952, 2, 3, 2452
+    seg = np.zeros((B, S), np.int32)
+    for c in (2262, 4065, 5165):
+        seg[0, c:] += 1
+    fn = ra.sliding_window_bias(window) + ra.segment_bias()
+    ofn = R.make_bias_fn(causal=True, window=window, use_segments=True)
+    for rep in range(3):
+        _against_dense_oracle(device, f"window edge inside a shard, documents, D={D}, call {rep}", B, S, H, D, n, fn, ofn,
+                              {"q_segment_ids": seg}, {"kv_segment_ids": seg}, seed=201060915)
