@@ -99,6 +99,56 @@ def test_long_shard_configurations(device, seed):
         _against_dense_oracle(device, f"long shards {seed}.{case} {kind} D={kw['D']} n={kw['n']} S={kw['S']}", **kw)
 
 
+def _ragged_cases(seed, count):
+    """Shard lengths on and off every grid of the kernels (200 ... 3000 tokens, 1-5 shards), batch 1-2,
+    1-3 heads, one to eight document cuts per batch row, windows from a few tokens to longer than the
+    sequence, and sums of the bias terms that the long-shard generator does not draw (two-sided
+    window + documents, ALiBi + window + documents, prefix-LM + documents)."""
+    for case in range(count):
+        rng = np.random.default_rng(seed * 1000 + case)
+        D, n, B, H = int(rng.choice([64, 128])), int(rng.choice([1, 2, 3, 4, 5])), int(rng.choice([1, 2])), int(rng.choice([1, 2, 3]))
+        L = int(rng.choice([200, 256, 320, 511, 777, 1000, 1024, 1111, 1536, 1984, 2048, 2500, 3000]))
+        while n * L > 7000:
+            n -= 1
+        S = n * L
+        kind = str(rng.choice(["window", "window2", "seg_causal", "seg", "alibi_seg", "alibi_causal_seg", "prefix", "window_seg",
+                               "window2_seg", "alibi_window_seg", "prefix_seg"]))
+        sl = R.alibi_slopes(H)
+        seg = np.zeros((B, S), np.int32)
+        for b in range(B):
+            for c in np.sort(rng.integers(0, S, int(rng.integers(1, 9)))):
+                seg[b, c:] += 1
+        w = int(rng.choice([rng.integers(1, 100), rng.integers(100, max(S // 2, 101)), rng.integers(max(S // 2, 101), S + 50)]))
+        segkw = ({"q_segment_ids": seg}, {"kv_segment_ids": seg})
+        pm = (np.arange(S)[None] < rng.integers(0, S, (B, 1))).astype(np.int32)
+        prekw = ({"q_prefix_mask": pm}, {"kv_prefix_mask": pm})
+        both = ({**segkw[0], **prekw[0]}, {**segkw[1], **prekw[1]})
+        fn, ofn, (qkw, kvkw) = {
+            "window": (ra.sliding_window_bias(w), R.make_bias_fn(causal=True, window=w), ({}, {})),
+            "window2": (ra.sliding_window_bias(w, causal=False), R.make_bias_fn(window=w), ({}, {})),
+            "seg_causal": (ra.segment_bias() + ra.causal_bias(), R.make_bias_fn(causal=True, use_segments=True), segkw),
+            "seg": (ra.segment_bias(), R.make_bias_fn(use_segments=True), segkw),
+            "alibi_seg": (ra.alibi_bias(sl) + ra.segment_bias(), R.make_bias_fn(use_segments=True, alibi=sl), segkw),
+            "alibi_causal_seg": (ra.alibi_bias(sl) + ra.causal_bias() + ra.segment_bias(),
+                                 R.make_bias_fn(causal=True, use_segments=True, alibi=sl), segkw),
+            "prefix": (ra.prefix_lm_bias(), R.make_bias_fn(use_prefix=True), prekw),
+            "window_seg": (ra.sliding_window_bias(w) + ra.segment_bias(),
+                           R.make_bias_fn(causal=True, window=w, use_segments=True), segkw),
+            "window2_seg": (ra.sliding_window_bias(w, causal=False) + ra.segment_bias(),
+                            R.make_bias_fn(window=w, use_segments=True), segkw),
+            "alibi_window_seg": (ra.alibi_bias(sl) + ra.sliding_window_bias(w) + ra.segment_bias(),
+                                 R.make_bias_fn(causal=True, window=w, use_segments=True, alibi=sl), segkw),
+            "prefix_seg": (ra.prefix_lm_bias() + ra.segment_bias(), R.make_bias_fn(use_prefix=True, use_segments=True), both),
+        }[kind]
+        yield f"ragged {seed}.{case} {kind} B={B} H={H} D={D} n={n} L={L} w={w}", dict(
+            B=B, S=S, H=H, D=D, n=n, fn=fn, ofn=ofn, qkw=qkw, kvkw=kvkw, seed=int(rng.integers(1 << 30)))
+
+
+def test_ragged_configurations(device):
+    for name, kw in _ragged_cases(7, 14):
+        _against_dense_oracle(device, name, **kw)
+
+
 @pytest.mark.parametrize("sm_scale", [1.0, 0.3, 0.02, 1e-3, 0.17])
 @pytest.mark.parametrize("D", [128, 64])
 def test_softmax_scales(device, sm_scale, D):
