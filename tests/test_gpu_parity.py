@@ -73,10 +73,10 @@ def _check(device, name, B, Sq, Sk, H, D, n, fn=None, ofn=None, qkw=None, kvkw=N
     want, want_lse = R.mha_dense(q, k, v, bias)
     np.testing.assert_array_equal(np.isnan(out), np.isnan(want))
     ok = ~np.isnan(want)
-    e_out, e_rel = np.abs(out - want)[ok].max(), _out_rel(out, want)
+    e_out, e_rel = np.abs(out - want)[ok].max(initial=0.0), _out_rel(out, want)
     okl = np.isfinite(want_lse)
     np.testing.assert_array_equal(np.isneginf(lse), np.isneginf(want_lse))
-    e_lse = np.abs(lse[okl] - want_lse[okl]).max()
+    e_lse = np.abs(lse[okl] - want_lse[okl]).max(initial=0.0)  # (no live query at all: nothing to compare)
     worst = {"out": e_out, "out_rel": e_rel, "lse": e_lse}
     assert e_out <= OUT_TOL and e_rel <= OUT_REL and e_lse <= LSE_TOL, worst
     if grads:
@@ -91,6 +91,8 @@ def _check(device, name, B, Sq, Sk, H, D, n, fn=None, ofn=None, qkw=None, kvkw=N
         for got, ref, nm in zip(g, R.mha_dense_grads(q, k, v, do, bias), ("dq", "dk", "dv")):
             if nm == "dq":
                 got, ref = got[live], ref[live]
+                if got.size == 0:
+                    continue
             else:
                 assert np.isfinite(got).all(), nm
             mx, fro = _rel(got, ref)
@@ -866,6 +868,16 @@ def test_random_configurations(device, seed):
     for case, kind, kw in _random_cases(seed, 12):
         for impl in ("hip", "hip_fused", "pallas"):
             _check(device, f"random {seed}.{case} {kind}", impl=impl, **kw)
+
+
+@pytest.mark.parametrize("impl", ["hip", "hip_fused"])
+def test_random_configuration_in_which_no_query_sees_a_key(device, impl):
+    """Case 3 of sweep seed 109: six queries against 800 keys under causal + segment + ALiBi
+    biases, and every query row is fully masked.  All outputs are NaN and all logsumexps -inf
+    (ring.py:134-135), dk and dv are zero, and there is no live row to compare dq on."""
+    case, kind, kw = [c for c in _random_cases(109, 4)][3]
+    assert (kw["Sq"], kw["Sk"], kind) == (6, 800, "alibi_causal_seg")
+    _check(device, f"random 109.{case} {kind}", impl=impl, **kw)
 
 
 # The cases of the seed-0 sweep with shard lengths off the tile grid (300, 520, 100 queries;
