@@ -309,6 +309,9 @@ def main():
                     help="no GPU work: turn the counter_collection.csv files of two rocprofv3 --pmc runs of this "
                          "script (FETCH_SIZE, WRITE_SIZE; both with --copy-probe) into the text summary kept "
                          "under profiles/ and print it")
+    ap.add_argument("--no-dense-summary", action="store_true",
+                    help="CALLABLE: hand the step kernels the dense blocks without their summaries (ra_dense_map), "
+                         "so that they read every block in full: the streaming rate of the dense-bias kernels")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain elementwise copy of 1 GiB (calibrates HBM byte counters)")
     ap.add_argument("--coissue-probe", action="store_true",
@@ -380,6 +383,10 @@ def main():
                 sid += 1
         seg = torch.from_numpy(seg_np).to(dev)
         if w["bias"] == "callable":
+            if args.no_dense_summary:
+                from ring_attention import bias as rbias
+                rbias.DENSE_SUMMARY = False
+
             def fn(q_segment_ids, kv_segment_ids):  # the form of ring_test.py:226-233, head-broadcast
                 same = q_segment_ids[:, :, None] == kv_segment_ids[:, None, :]
                 return torch.where(same, 0.0, float("-inf"))[:, None]
@@ -558,7 +565,23 @@ def main():
                 "algorithmic_tflop_per_launch": round(d["flops"] / d["launches"] / 1e12, 4),
                 "achieved_tflops": round(d["flops"] / d["ms"] / 1e9, 2)}
         dom = max(kern, key=lambda kk: kern[kk]["ms"])
-        if w["bias"] == "callable":
+        if w["bias"] == "callable" and not args.no_dense_summary:
+            # Every block goes through one summary pass (ra_dense_map, inside the forward launch's
+            # bracket and again in the backward step's: the callable is called once per loop,
+            # ring.py:107,186); the step kernels then leave out what is -inf throughout and read the
+            # block only where it is not zero: matrix work over the unmasked pairs, as in the other
+            # workloads.
+            ach = kern[dom]["flops"] / kern[dom]["ms"] / 1e9
+            result["roofline"] = {"bound": "mfma", "kernel": names[dom] + "<D, 2> with the block's summary",
+                                  "achieved": round(ach, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                  "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None}
+            for kind in kern:
+                ev_ = [ms for (k2, qs, ks), ms in recs if k2 == kind]
+                kernels[names[kind]]["avg_ms_all_launches"] = round(sum(ev_) / len(ev_), 4)
+            k_ms = sum(ms for _, ms in recs)
+            result["host_and_torch_ms_per_step"] = round(ms_per_step - k_ms, 3)
+            result["step_kernels_ms_per_step"] = round(k_ms, 3)
+        elif w["bias"] == "callable":
             # the kernels stream the dense [b, 1, lq, lk] fp32 block: 4 bytes per (query, key) position
             # and launch if the heads of a launch share one pass over it, next to which the bf16
             # operands and fp32 carries of the step are small: HBM bound

@@ -118,6 +118,15 @@ typedef struct ra_bias {
    * other terms by addition.  No gradient is produced for it (ring.py:243 returns None). */
   const float* dense_bias;
   int64_t dense_stride_b, dense_stride_h, dense_stride_q;
+  /* Optional (NULL: none) with RA_BIAS_DENSE: the block's summary as written by ra_dense_map().
+   * The reference hands its kernels the whole block and they read all of it
+   * (ring_kernel.py:75-85); the blocks a bias_fn returns are mostly masks (ring_test.py:226-246:
+   * 0 or -inf), so ra_fwd_step / ra_bwd_step take the summary to leave out the tiles whose part of
+   * the block is -inf throughout (they contribute exp(-inf) = 0, exactly) and to read the block
+   * only in tiles that hold a value other than 0.  Results are those without a summary.  It must
+   * describe this block (same strides and shape); the several-step entry points evaluate the
+   * whole block and do not read it.  Shards of at most RA_MAX_SEGMENT_SHARD tokens. */
+  const uint8_t* dense_map;
 } ra_bias;
 
 /* One ring step of the forward pass. */
@@ -270,6 +279,18 @@ int ra_bwd_delta_passes(const void* out, int32_t out_dtype, int64_t out_stride_p
 int ra_bwd_finalize_passes(const float* acc, void* out, int64_t out_stride_pass, int64_t out_stride_b,
                            int64_t out_stride_h, int64_t out_stride_l, int32_t n_passes, int32_t B,
                            int32_t H, int32_t L, int32_t D, void* stream);
+
+/* Summary of a dense bias block for ra_bias.dense_map: one byte per cell of 32 queries x 32 keys,
+ * bit 0 = the cell holds a value other than -inf, bit 1 = it holds a value other than 0;
+ * map[nb, nh, ceil(Lq/32), ceil(Lk/32)] with nb = B (1 if stride_b is 0) and nh = H (1 if
+ * stride_h is 0), ra_dense_map_bytes() bytes.  One pass over the block (HBM bound), to be run
+ * once per block that a bias_fn returns (ring.py:107,186: the reference calls bias_fn once per
+ * ring step in the forward and once more in the backward loop); the forward step and both halves
+ * of the backward step of the pair then share it.  B, H, Lq, Lk and the strides are those of the
+ * step the block belongs to. */
+int64_t ra_dense_map_bytes(int64_t stride_b, int64_t stride_h, int32_t B, int32_t H, int32_t Lq, int32_t Lk);
+int ra_dense_map(const float* dense_bias, int64_t stride_b, int64_t stride_h, int64_t stride_q, int32_t B,
+                 int32_t H, int32_t Lq, int32_t Lk, uint8_t* map, void* stream);
 
 /* Host-only, pure: 1 if every score of the (query shard, key/value shard) pair is masked
  * by the positional terms of `bias` (CAUSAL / WINDOW), so that the whole ring step is an

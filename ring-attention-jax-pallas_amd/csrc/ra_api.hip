@@ -88,6 +88,8 @@ int check_bias(const ra_bias& b, int Lq, int Lk) {
     if (b.dense_stride_q < Lk || b.dense_stride_b < 0 || b.dense_stride_h < 0)
       return fail(RA_ERR_BIAS, "dense bias strides: stride_q must be at least Lk, stride_b / stride_h "
                                "non-negative (0 broadcasts)");
+    if (b.dense_map && (Lq > kMaxSegLen || Lk > kMaxSegLen))
+      return fail(RA_ERR_SHAPE, "a dense bias with its summary supports shards of at most %d tokens", kMaxSegLen);
   }
   if (b.q_offset < 0 || b.kv_offset < 0 || b.q_offset + Lq > kMaxPos || b.kv_offset + Lk > kMaxPos)
     return fail(RA_ERR_BIAS, "token positions (offset + index) must lie in [0, 2^30 - 2^16)");
@@ -117,6 +119,7 @@ ra::BiasArgs to_bias(const ra_bias& b) {
   r.dense_sb = b.dense_stride_b;
   r.dense_sh = b.dense_stride_h;
   r.dense_sq = b.dense_stride_q;
+  r.dense_map = (b.flags & RA_BIAS_DENSE) ? b.dense_map : nullptr;
   return r;
 }
 
@@ -529,7 +532,7 @@ int bwd_dkdv_passes(const ra_bwd_step_params* steps, const std::vector<int>& fir
 
 extern "C" {
 
-int ra_version(void) { return 1005; }
+int ra_version(void) { return 1006; }
 
 const char* ra_last_error(void) { return g_err; }
 
@@ -583,6 +586,30 @@ int ra_fwd_init(float* o, float* m, float* l, int32_t B, int32_t H, int32_t Lq, 
   if (rc) return rc;
   hipError_t e = ra::launch_fwd_init(o, m, l, (long long)B * H * Lq, D, (hipStream_t)stream);
   return e == hipSuccess ? RA_OK : hip_fail(e, "ra_fwd_init launch");
+}
+
+int64_t ra_dense_map_bytes(int64_t stride_b, int64_t stride_h, int32_t B, int32_t H, int32_t Lq, int32_t Lk) {
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0) return 0;
+  const int64_t cells = (int64_t)((Lq + 31) / 32) * ((Lk + 31) / 32);
+  return (stride_b ? B : 1) * (int64_t)(stride_h ? H : 1) * cells;
+}
+
+int ra_dense_map(const float* dense_bias, int64_t stride_b, int64_t stride_h, int64_t stride_q, int32_t B,
+                 int32_t H, int32_t Lq, int32_t Lk, uint8_t* map, void* stream) {
+  if (!dense_bias || !map) return fail(RA_ERR_NULL, "ra_dense_map: NULL pointer");
+  if (B <= 0 || H <= 0 || Lq <= 0 || Lk <= 0)
+    return fail(RA_ERR_SHAPE, "ra_dense_map: bad shape B=%d H=%d Lq=%d Lk=%d", B, H, Lq, Lk);
+  if (Lq > kMaxSegLen || Lk > kMaxSegLen)
+    return fail(RA_ERR_SHAPE, "ra_dense_map: shards of at most %d tokens", kMaxSegLen);
+  if (((uintptr_t)dense_bias & 3) != 0) return fail(RA_ERR_ALIGN, "dense_bias is not 4-byte aligned");
+  if (stride_q < Lk || stride_b < 0 || stride_h < 0)
+    return fail(RA_ERR_BIAS, "dense bias strides: stride_q must be at least Lk, stride_b / stride_h "
+                             "non-negative (0 broadcasts)");
+  const int nb = stride_b ? B : 1, nh = stride_h ? H : 1;
+  if ((int64_t)nb * nh > 65535) return fail(RA_ERR_SHAPE, "ra_dense_map: more than 65535 (batch, head) blocks");
+  hipError_t e = ra::launch_dense_map(dense_bias, stride_b, stride_h, stride_q, nb, nh, Lq, Lk, map,
+                                      (hipStream_t)stream);
+  return e == hipSuccess ? RA_OK : hip_fail(e, "ra_dense_map launch");
 }
 
 int ra_fwd_step(const ra_fwd_step_params* p, void* stream) {

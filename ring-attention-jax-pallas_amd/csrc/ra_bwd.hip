@@ -255,31 +255,52 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   bool wg_one_doc = true;
   const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
   const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
-  if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
+  // A dense block that comes with its summary is listed the same way: tiles in which the
+  // workgroup's keys meet nothing but -inf are left out, tiles of zeros have no term to evaluate,
+  // the rest is evaluated element by element.  (Single-step launches only.)
+  const unsigned char* dmap = nullptr;
+  if constexpr (DENSE && !MULTI) {
+    if (bs.dense_map) dmap = dense_map_of(bs, b, h, a.H, a.Lq, a.Lk);
+  }
+  if ((GENERAL && (flags & RA_BIAS_SEGMENT)) || (DENSE && dmap != nullptr)) {
     use_list = true;
-    int smin = 0x7fffffff, smax = (int)0x80000000;
-    if (kw + l32 < a.Lk) {
-      smin = k_seg;
-      smax = k_seg;
-    }
-    smin = wave_min(smin);
-    smax = wave_max(smax);
-    if (lane == 0) {
-      s_red[wave] = smin;
-      s_red[4 + wave] = smax;
-    }
-    __syncthreads();
-    int kmin = s_red[0], kmax = s_red[4];
+    int kmin = 0, kmax = 0;
+    if (seg_on) {
+      int smin = 0x7fffffff, smax = (int)0x80000000;
+      if (kw + l32 < a.Lk) {
+        smin = k_seg;
+        smax = k_seg;
+      }
+      smin = wave_min(smin);
+      smax = wave_max(smax);
+      if (lane == 0) {
+        s_red[wave] = smin;
+        s_red[4 + wave] = smax;
+      }
+      __syncthreads();
+      kmin = s_red[0];
+      kmax = s_red[4];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) {
-      kmin = min(kmin, s_red[w]);
-      kmax = max(kmax, s_red[4 + w]);
+      for (int w = 1; w < 4; ++w) {
+        kmin = min(kmin, s_red[w]);
+        kmax = max(kmax, s_red[4 + w]);
+      }
     }
     for (int i = i_lo + tid; i < i_hi; i += NT) {
-      int qmin, qmax;
-      tile_id_range<kQTile>(q_seg, i, a.Lq, qmin, qmax);
-      const bool act = !(qmax < kmin || qmin > kmax);
-      s_flag[i - i_lo] = act ? ((qmin == qmax) ? 1 : 3) : 0;
+      int f = 1;
+      if (seg_on) {
+        int qmin, qmax;
+        tile_id_range<kQTile>(q_seg, i, a.Lq, qmin, qmax);
+        const bool act = !(qmax < kmin || qmin > kmax);
+        f = act ? ((qmin == qmax) ? 1 : 3) : 0;
+      }
+      if constexpr (DENSE) {
+        if (dmap != nullptr && f != 0) {
+          const int bits = dense_map_or(dmap, a.Lk, i * kQTile, min((i + 1) * kQTile, a.Lq) - 1, k0, k_hi);
+          f = (bits & kMapLive) ? ((bits & kMapNonZero) ? 3 : f) : 0;
+        }
+      }
+      s_flag[i - i_lo] = f;
     }
     wg_one_doc = kmin == kmax;
     __syncthreads();
@@ -458,9 +479,15 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     return classify_pos(flags, bs.window, q_off + qt0, q_off + qt0 + kQTile - 1, kv_off + kw,
                         kv_off + kw + 31);
   };
+  // terms that every tile must evaluate; a dense block with a summary is read only in the tiles
+  // that the list marks (segbit)
+  int tile_terms = RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE;
+  if constexpr (DENSE) {
+    if (dmap != nullptr) tile_terms &= ~RA_BIAS_DENSE;
+  }
   auto needs_bias = [&](int qt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (qt0 + kQTile > a.Lq);
-    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
+    if (GENERAL) nb = nb || (flags & tile_terms) || segbit;
     return nb;
   };
   constexpr int PFN = 4;  // operand fetches kept in flight ahead of the MFMA that uses them
@@ -511,8 +538,8 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
-      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE);
-      if (segbit) tb.flags |= RA_BIAS_SEGMENT;
+      tb.flags |= flags & tile_terms;
+      if (segbit) tb.flags |= DENSE ? (flags & (RA_BIAS_SEGMENT | RA_BIAS_DENSE)) : RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
@@ -552,7 +579,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
   int plain_lo = 0, plain_hi = 0;
   if constexpr (GENERAL) {
     int st_lo[4] = {0, 0, 0, 0}, st_hi[4] = {0, 0, 0, 0};
-    if (wave_on && !(flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE))) {
+    if (wave_on && !(flags & tile_terms & (RA_BIAS_PREFIX | RA_BIAS_DENSE))) {
       int lo, hi;
       query_tile_plain_range(flags, bs.window, kv_off + kw, kv_off + kw + 31, q_off, a.Lq / kQTile,
                              kQTile, lo, hi);
@@ -898,7 +925,7 @@ __global__ __launch_bounds__(256) void dkdv_kernel(
     plain_iteration(P4{}, i + 4, s_a, p_a, s_b, p_b);
     plain_iteration(P5{}, i + 5, s_b, p_b, s_a, p_a);
   }
-  } else if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+  } else {
 #pragma unroll 1
   for (int st = 0; st < 4; ++st) {
     // iteration i is plain for p_lo < i < p_end
@@ -1223,27 +1250,48 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   int cons_hi = n_act, cons2_hi = 0;
   bool wg_one_doc = true;
   const bool seg_on = GENERAL && (flags & RA_BIAS_SEGMENT);
-  if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
+  // A dense block that comes with its summary is listed the same way: tiles in which the
+  // workgroup's rows hold nothing but -inf are left out, tiles of zeros have no term to evaluate,
+  // the rest is evaluated element by element.  (Single-step launches only.)
+  const unsigned char* dmap = nullptr;
+  if constexpr (DENSE && !MULTI) {
+    if (bs.dense_map) dmap = dense_map_of(bs, b, h, a.H, a.Lq, a.Lk);
+  }
+  if ((GENERAL && (flags & RA_BIAS_SEGMENT)) || (DENSE && dmap != nullptr)) {
     use_list = true;
-    int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
-    smin = wave_min(smin);
-    smax = wave_max(smax);
-    if (lane == 0) {
-      s_red[wave] = smin;
-      s_red[8 + wave] = smax;
-    }
-    __syncthreads();
-    int qmin = s_red[0], qmax = s_red[8];
+    int qmin = 0, qmax = 0;
+    if (seg_on) {
+      int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
+      smin = wave_min(smin);
+      smax = wave_max(smax);
+      if (lane == 0) {
+        s_red[wave] = smin;
+        s_red[8 + wave] = smax;
+      }
+      __syncthreads();
+      qmin = s_red[0];
+      qmax = s_red[8];
 #pragma unroll
-    for (int w = 1; w < 8; ++w) {
-      qmin = min(qmin, s_red[w]);
-      qmax = max(qmax, s_red[8 + w]);
+      for (int w = 1; w < 8; ++w) {
+        qmin = min(qmin, s_red[w]);
+        qmax = max(qmax, s_red[8 + w]);
+      }
     }
     for (int j = j_lo + tid; j < j_hi; j += kDqThreads) {
-      int kmin, kmax;
-      tile_id_range<kDqKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
-      const bool act = !(kmax < qmin || kmin > qmax);
-      s_flag[j - j_lo] = act ? ((kmin == kmax) ? 1 : 3) : 0;
+      int f = 1;
+      if (seg_on) {
+        int kmin, kmax;
+        tile_id_range<kDqKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
+        const bool act = !(kmax < qmin || kmin > qmax);
+        f = act ? ((kmin == kmax) ? 1 : 3) : 0;
+      }
+      if constexpr (DENSE) {
+        if (dmap != nullptr && f != 0) {
+          const int bits = dense_map_or(dmap, a.Lk, q0, q_rows_hi, j * kDqKeyTile, min((j + 1) * kDqKeyTile, a.Lk) - 1);
+          f = (bits & kMapLive) ? ((bits & kMapNonZero) ? 3 : f) : 0;
+        }
+      }
+      s_flag[j - j_lo] = f;
     }
     wg_one_doc = qmin == qmax;
     __syncthreads();
@@ -1377,9 +1425,15 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     return classify_pos(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off + kt0,
                         kv_off + kt0 + kDqKeyTile - 1);
   };
+  // terms that every tile must evaluate; a dense block with a summary is read only in the tiles
+  // that the list marks (segbit)
+  int tile_terms = RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE;
+  if constexpr (DENSE) {
+    if (dmap != nullptr) tile_terms &= ~RA_BIAS_DENSE;
+  }
   auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (kt0 + kDqKeyTile > a.Lk);
-    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
+    if (GENERAL) nb = nb || (flags & tile_terms) || segbit;
     return nb;
   };
   constexpr int PF = 2;
@@ -1425,8 +1479,8 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
-      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE);
-      if (segbit) tb.flags |= RA_BIAS_SEGMENT;
+      tb.flags |= flags & tile_terms;
+      if (segbit) tb.flags |= DENSE ? (flags & (RA_BIAS_SEGMENT | RA_BIAS_DENSE)) : RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     tb.slope2 = slope2;
@@ -1474,7 +1528,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
   const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
   if constexpr (GENERAL) {
     int st_lo[4] = {0, 0, 0, 0}, st_hi[4] = {0, 0, 0, 0};
-    if (wave_on && lse_in_range && !(flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE))) {
+    if (wave_on && lse_in_range && !(flags & tile_terms & (RA_BIAS_PREFIX | RA_BIAS_DENSE))) {
       int lo, hi;
       key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kDqKeyTile,
                            kDqKeyTile, lo, hi);
@@ -1824,7 +1878,7 @@ __global__ __launch_bounds__(kDqThreads) void dq_kernel(
       delta = s_rowc[1][tid];
     }
   }
-  } else if constexpr (!DENSE) {  // a dense bias block leaves no plain stretch
+  } else {
 #pragma unroll 1
   for (int st = 0; st < 4; ++st) {
     // iteration i is plain for p_lo < i < p_end

@@ -40,7 +40,30 @@ struct BiasArgs {
   const float* slopes;
   const float* dense;  // additive bias block [B|1, H|1, Lq, Lk], keys contiguous
   long long dense_sb, dense_sh, dense_sq;
+  // optional summary of the block, one byte per cell of 32 queries x 32 keys (dense_map_kernel):
+  // bit 0 = the cell holds a value other than -inf, bit 1 = it holds a value other than 0;
+  // [B|1, H|1, ceil(Lq / 32), ceil(Lk / 32)], broadcast like the block itself
+  const unsigned char* dense_map;
 };
+
+constexpr int kMapCell = 32;  // queries and keys per cell of a dense block's summary
+constexpr int kMapLive = 1, kMapNonZero = 2;
+
+// The summary's rows of one (batch, head) and the OR over a rectangle of its cells: what a
+// workgroup needs to know about the part of the block that its rows and one tile span.
+RA_DEV const unsigned char* dense_map_of(const BiasArgs& bs, int b, int h, int H, int Lq, int Lk) {
+  const long long cells = (long long)((Lq + kMapCell - 1) / kMapCell) * ((Lk + kMapCell - 1) / kMapCell);
+  const long long hm = bs.dense_sh ? H : 1;
+  return bs.dense_map + ((bs.dense_sb ? b : 0) * hm + (bs.dense_sh ? h : 0)) * cells;
+}
+RA_DEV int dense_map_or(const unsigned char* mp, int Lk, int q_lo, int q_hi, int k_lo, int k_hi) {
+  // queries [q_lo, q_hi] x keys [k_lo, k_hi], inclusive and in range
+  const int ncols = (Lk + kMapCell - 1) / kMapCell;
+  int bits = 0;
+  for (int r = q_lo / kMapCell; r <= q_hi / kMapCell; ++r)
+    for (int c = k_lo / kMapCell; c <= k_hi / kMapCell; ++c) bits |= mp[(long long)r * ncols + c];
+  return bits;
+}
 
 struct TensorArg {
   const bf16_t* ptr;
@@ -232,6 +255,8 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
   const bool causal = flags & RA_BIAS_CAUSAL, window = flags & RA_BIAS_WINDOW;
   const bool segment = flags & RA_BIAS_SEGMENT, prefix = flags & RA_BIAS_PREFIX;
   const bool dense_vec = DENSE && __builtin_amdgcn_readfirstlane(tb.dense_vec) != 0;
+  // the block is read for this tile (always, unless its summary says that the tile holds zeros)
+  const bool dense_on = DENSE && (flags & RA_BIAS_DENSE);
   int lo = 0, hi = tb.var_limit - 1;  // off >= var_limit: out of range
   int pre_lo = -kFar, pre_hi = kFar;  // outside [pre_lo, pre_hi]: rel < 0, masked unless both sides are prefix
   // |rel0| < 2^30 and window <= 2^30 (the host checks positions and clamps the window), so the sums
@@ -267,7 +292,7 @@ RA_DEV void apply_bias(f32x16& t, const TileBias& tb, int rel0, int fixed_seg, i
       if (segment) vs = *(const i32x4*)(var_seg + 8 * bb);
       if (PRE) vp = *(const i32x4*)(var_pre + 8 * bb);
       float dn[4] = {0.f, 0.f, 0.f, 0.f};
-      if (DENSE) {
+      if (DENSE && dense_on) {
         if (QFIXED && dense_vec) {
           // a lane's four keys are 16 contiguous bytes of its row: one load instead of four
           const f32x4 v4 = *(const f32x4*)(tb.dense + 8 * bb);

@@ -203,29 +203,52 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // the listed tiles count up without a gap from the start of a run to ordinal cons_hi / cons2_hi
   int cons_hi = n_act, cons2_hi = 0;
   bool wg_one_doc = true;
-  if (GENERAL && (flags & RA_BIAS_SEGMENT)) {
+  // A dense block that comes with its summary is listed the same way: tiles in which the
+  // workgroup's rows hold nothing but -inf are left out, tiles of zeros count as tiles of one
+  // id (no term to evaluate: they may join a straight-line stretch), the rest is evaluated
+  // element by element.  (Single-step launches only.)
+  const unsigned char* dmap = nullptr;
+  if constexpr (DENSE && !MULTI) {
+    if (bs.dense_map) dmap = dense_map_of(bs, b, h, a.H, a.Lq, a.Lk);
+  }
+  const bool seg_list = GENERAL && (flags & RA_BIAS_SEGMENT);
+  if (seg_list || (DENSE && dmap != nullptr)) {
     // segment-id range of the workgroup's queries, then one thread per key tile decides
     // whether the id ranges can intersect (skip otherwise) and whether the tile has one id
     use_list = true;
-    int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
-    smin = wave_min(smin);
-    smax = wave_max(smax);
-    if (lane == 0) {
-      s_red[wave] = smin;
-      s_red[8 + wave] = smax;
-    }
-    __syncthreads();
-    int qmin = s_red[0], qmax = s_red[8];
+    int qmin = 0, qmax = 0;
+    if (seg_list) {
+      int smin = q_valid ? q_seg : 0x7fffffff, smax = q_valid ? q_seg : (int)0x80000000;
+      smin = wave_min(smin);
+      smax = wave_max(smax);
+      if (lane == 0) {
+        s_red[wave] = smin;
+        s_red[8 + wave] = smax;
+      }
+      __syncthreads();
+      qmin = s_red[0];
+      qmax = s_red[8];
 #pragma unroll
-    for (int w = 1; w < 8; ++w) {
-      qmin = min(qmin, s_red[w]);
-      qmax = max(qmax, s_red[8 + w]);
+      for (int w = 1; w < 8; ++w) {
+        qmin = min(qmin, s_red[w]);
+        qmax = max(qmax, s_red[8 + w]);
+      }
     }
     for (int j = j_lo + tid; j < j_hi; j += kFwdThreads) {
-      int kmin, kmax;
-      tile_id_range<kKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
-      const bool act = !(kmax < qmin || kmin > qmax);
-      s_flag[j - j_lo] = act ? ((kmin == kmax) ? 1 : 3) : 0;
+      int f = 1;
+      if (seg_list) {
+        int kmin, kmax;
+        tile_id_range<kKeyTile>(kv_seg, j, a.Lk, kmin, kmax);
+        const bool act = !(kmax < qmin || kmin > qmax);
+        f = act ? ((kmin == kmax) ? 1 : 3) : 0;
+      }
+      if constexpr (DENSE) {
+        if (dmap != nullptr && f != 0) {
+          const int bits = dense_map_or(dmap, a.Lk, q0, q_rows_hi, j * kKeyTile, min((j + 1) * kKeyTile, a.Lk) - 1);
+          f = (bits & kMapLive) ? ((bits & kMapNonZero) ? 3 : f) : 0;
+        }
+      }
+      s_flag[j - j_lo] = f;
     }
     wg_one_doc = qmin == qmax;
     __syncthreads();
@@ -513,9 +536,15 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, S[kb][r]);
     return half_max(mx) * a.scale2;  // scale2 > 0: the maximum commutes with the scaling
   };
+  // terms that every tile must evaluate; a dense block with a summary is read only in the tiles
+  // that the list marks (segbit)
+  int tile_terms = RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE;
+  if constexpr (DENSE) {
+    if (dmap != nullptr) tile_terms &= ~RA_BIAS_DENSE;
+  }
   auto needs_bias = [&](int kt0, int segbit, int cls) -> bool {
     bool nb = (cls & 2) || (kt0 + kKeyTile > a.Lk);
-    if (GENERAL) nb = nb || (flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE)) || segbit;
+    if (GENERAL) nb = nb || (flags & tile_terms) || segbit;
     return nb;
   };
   // Bias of a fresh tile with the id arrays of LDS slot `ids_buf`; returns the row maximum (log2
@@ -525,8 +554,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     TileBias tb;
     tb.flags = (cls & 2) ? (flags & (RA_BIAS_CAUSAL | RA_BIAS_WINDOW)) : 0;
     if (GENERAL) {
-      tb.flags |= flags & (RA_BIAS_ALIBI | RA_BIAS_PREFIX | RA_BIAS_DENSE);
-      if (segbit) tb.flags |= RA_BIAS_SEGMENT;
+      tb.flags |= flags & tile_terms;
+      if (segbit) tb.flags |= DENSE ? (flags & (RA_BIAS_SEGMENT | RA_BIAS_DENSE)) : RA_BIAS_SEGMENT;
     }
     tb.window = bs.window;
     const float inv_scale2 = 1.0f / a.scale2;
@@ -581,7 +610,7 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   constexpr int NST = 4;
   const bool alibi_on = GENERAL && (flags & RA_BIAS_ALIBI);
   int st_lo[NST] = {0, 0, 0, 0}, st_hi[NST] = {0, 0, 0, 0};
-  if (wave_on && !(GENERAL && (flags & (RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
+  if (wave_on && !(GENERAL && (flags & tile_terms & (RA_BIAS_PREFIX | RA_BIAS_DENSE)))) {
     int lo, hi;  // tile indices
     key_tile_plain_range(flags, bs.window, q_off + qw, q_off + qw + 31, kv_off, a.Lk / kKeyTile,
                          kKeyTile, lo, hi);
@@ -1229,6 +1258,49 @@ __global__ void fwd_init_kernel(float* o, float* m, float* l, long long rows, in
   }
 }
 
+// Summary of a dense bias block [nb, nh, Lq, Lk] (the strides say where a batch / head starts):
+// one byte per cell of 32 queries x 32 keys, bit 0 = some value of the cell is not -inf, bit 1 =
+// some value is not 0 (elements beyond Lq / Lk count for nothing).  A wave takes 32 rows x 256
+// keys, eight cells: lane l reads keys 4l .. 4l+3 of every row.  HBM bound: the block is read once.
+__global__ __launch_bounds__(256) void dense_map_kernel(const float* dense, long long sb, long long sh,
+                                                        long long sq, int nh, int Lq, int Lk, unsigned char* map) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ncols = (Lk + kMapCell - 1) / kMapCell, nrows = (Lq + kMapCell - 1) / kMapCell;
+  const int cg = blockIdx.x * 4 + wave;  // group of eight cell columns
+  const int rb = blockIdx.y, bh = blockIdx.z;
+  if (cg * 8 >= ncols) return;
+  const float* base = dense + (bh / nh) * sb + (bh % nh) * sh;
+  const int k0 = cg * 256 + 4 * lane;
+  const bool vec = k0 + 3 < Lk && ((((uintptr_t)base) | ((uintptr_t)sq << 2)) & 15) == 0;
+  const int rows = min(kMapCell, Lq - rb * kMapCell);
+  bool live = false, nonzero = false;
+#pragma unroll 4
+  for (int r = 0; r < rows; ++r) {
+    const float* p = base + (long long)(rb * kMapCell + r) * sq + k0;
+    float x[4] = {RA_NEG_INF, RA_NEG_INF, RA_NEG_INF, RA_NEG_INF};
+    if (vec) {
+      const f32x4 v = *(const f32x4*)p;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) x[c] = v[c];
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (k0 + c < Lk) x[c] = p[c];
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const bool in = vec || k0 + c < Lk;
+      live |= in && !(x[c] == RA_NEG_INF);
+      nonzero |= in && x[c] != 0.f;
+    }
+  }
+  const unsigned long long ml = __ballot(live), mn = __ballot(nonzero);
+  if (lane < 8 && cg * 8 + lane < ncols) {
+    const int bits = (((ml >> (8 * lane)) & 0xffull) ? kMapLive : 0) | (((mn >> (8 * lane)) & 0xffull) ? kMapNonZero : 0);
+    map[((long long)bh * nrows + rb) * ncols + cg * 8 + lane] = (unsigned char)bits;
+  }
+}
+
 // The carries of n_pass query shards lie one after another ([n_pass, B, H, Lq, D]); shard p is
 // written to out + p * sp.
 template <typename OutT>
@@ -1293,6 +1365,14 @@ hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, 
   const long long n = rows * (D / 4);
   hipLaunchKernelGGL(fwd_init_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, o, m, l,
                      rows, D);
+  return hipGetLastError();
+}
+
+hipError_t launch_dense_map(const float* dense, long long sb, long long sh, long long sq, int nb, int nh, int Lq,
+                            int Lk, unsigned char* map, hipStream_t stream) {
+  const int ncols = (Lk + kMapCell - 1) / kMapCell, nrows = (Lq + kMapCell - 1) / kMapCell;
+  dim3 grid((unsigned)((ncols + 31) / 32), (unsigned)nrows, (unsigned)(nb * nh));
+  hipLaunchKernelGGL(dense_map_kernel, grid, dim3(256), 0, stream, dense, sb, sh, sq, nh, Lq, Lk, map);
   return hipGetLastError();
 }
 

@@ -106,6 +106,8 @@ struct QRing {
 hipError_t launch_fwd_step(const FwdArgs& a, int D, int mode, hipStream_t stream);
 hipError_t launch_fwd_steps(const FwdArgs& a, const KvRing& ring, int D, int mode, hipStream_t stream);
 hipError_t launch_fwd_init(float* o, float* m, float* l, long long rows, int D, hipStream_t stream);
+hipError_t launch_dense_map(const float* dense, long long sb, long long sh, long long sq, int nb, int nh, int Lq,
+                            int Lk, unsigned char* map, hipStream_t stream);
 hipError_t launch_fwd_finalize(const float* o, const float* m, const float* l, void* out, int out_f32,
                                long long sp, long long sb, long long sh, long long sl, float* lse, int n_pass,
                                int B, int H, int Lq, int D, hipStream_t stream);

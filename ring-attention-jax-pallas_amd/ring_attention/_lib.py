@@ -38,6 +38,7 @@ class RaBias(C.Structure):
         ("alibi_slopes", C.c_void_p),
         ("dense_bias", C.c_void_p),
         ("dense_stride_b", C.c_int64), ("dense_stride_h", C.c_int64), ("dense_stride_q", C.c_int64),
+        ("dense_map", C.c_void_p),
     ]
 
 
@@ -98,6 +99,9 @@ EXPORTS = {
                                          C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
     "ra_bwd_finalize": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32,
                                   C.c_int32, C.c_int32, C.c_int32, C.c_void_p]),
+    "ra_dense_map_bytes": (C.c_int64, [C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "ra_dense_map": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.c_int32, C.c_int32,
+                               C.c_int32, C.c_void_p, C.c_void_p]),
     "ra_step_is_skippable": (C.c_int, [C.POINTER(RaBias), C.c_int32, C.c_int32]),
     "ra_fwd_step_check": (C.c_int, [C.POINTER(RaFwdStepParams)]),
     "ra_bwd_step_check": (C.c_int, [C.POINTER(RaBwdStepParams)]),

@@ -29,6 +29,10 @@ import torch
 
 from . import _lib
 
+# A dense block is handed to the single-step launches together with its summary (one more pass
+# over the block, shared by the three kernels of the pair); False: the kernels read all of it.
+DENSE_SUMMARY = True
+
 
 @dataclass(frozen=True)
 class BiasFn:
@@ -129,7 +133,9 @@ class BlockBias:
     # its fwd_block / bwd_block take (ring.py:107, ring_kernel.py:127); added to the other terms
     dense: Optional[torch.Tensor] = None
 
-    def to_struct(self, device) -> "_lib.RaBias":
+    def to_struct(self, device, summary: bool = True) -> "_lib.RaBias":
+        """``summary``: hand a dense block's summary along (built once per block and kept with
+        it: the forward step and both halves of the backward step of a pair share it)."""
         s = _lib.RaBias()
         fn = self.fn
         s.flags = fn.flags
@@ -174,7 +180,27 @@ class BlockBias:
             s.dense_stride_b = 0 if d.shape[0] == 1 else d.stride(0)
             s.dense_stride_h = 0 if d.shape[1] == 1 else d.stride(1)
             s.dense_stride_q = d.stride(2)
+            if summary and DENSE_SUMMARY and d.is_cuda and max(d.shape[2], d.shape[3]) <= _lib.RA_MAX_SEGMENT_SHARD:
+                s.dense_map = self._dense_summary(d, s).data_ptr()
         return s
+
+    def _dense_summary(self, d: torch.Tensor, s: "_lib.RaBias") -> torch.Tensor:
+        """One byte per 32 x 32 cell of the block (``ra_dense_map``): the step kernels leave out
+        tiles that are -inf throughout and read the block only where it is not zero."""
+        key = (d.data_ptr(), tuple(d.shape), tuple(d.stride()), d._version)
+        hit = self.__dict__.get("_summary")
+        if hit is None or hit[0] != key:
+            lib = _lib.load()
+            B, H, Lq, Lk = d.shape
+            size = lib.ra_dense_map_bytes(s.dense_stride_b, s.dense_stride_h, B, H, Lq, Lk)
+            m = torch.empty((size,), dtype=torch.uint8, device=d.device)
+            stream = torch.cuda.current_stream(d.device).cuda_stream
+            _lib.check("ra_dense_map", lib.ra_dense_map(d.data_ptr(), s.dense_stride_b, s.dense_stride_h,
+                                                        s.dense_stride_q, B, H, Lq, Lk, m.data_ptr(), stream))
+            hit = (key, m, d)
+            self.__dict__["_summary"] = hit
+        self._keep.append(hit[1])
+        return hit[1]
 
     def check_dense_shape(self, B: int, H: int, Lq: int, Lk: int) -> None:
         """The broadcasting rule of the reference's block functions: [b, h | 1, lq, lk]

@@ -124,16 +124,18 @@ def _kernel_ready(t: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------------------
 # block-level API (one ring step)
 # --------------------------------------------------------------------------------------
-def _bias_struct(bias, device, shape=None) -> _lib.RaBias:
+def _bias_struct(bias, device, shape=None, summary=True) -> _lib.RaBias:
     """``bias`` is None, a ``BlockBias`` or a dense additive array ``[b, h | 1, lq, lk]`` - the
-    form the reference's block functions take (ring_kernel.py:127,206)."""
+    form the reference's block functions take (ring_kernel.py:127,206).  ``summary``: a dense
+    block travels with its summary (``ra_dense_map``); the single-step launches read it, the
+    several-step launches do not, so their callers pass False."""
     if bias is None:
         return _lib.RaBias()
     if isinstance(bias, torch.Tensor):
         bias = BlockBias(dense=bias)
     if shape is not None:
         bias.check_dense_shape(*shape)
-    return bias.to_struct(device)
+    return bias.to_struct(device, summary=summary)
 
 
 def fwd_block(q, k, v, bias: Union[BlockBias, torch.Tensor, None], o, m, l, sm_scale: float):
@@ -161,7 +163,7 @@ def fwd_block(q, k, v, bias: Union[BlockBias, torch.Tensor, None], o, m, l, sm_s
     return o, m, l
 
 
-def _fwd_params(q, k, v, bias, o, m, l, sm_scale) -> _lib.RaFwdStepParams:
+def _fwd_params(q, k, v, bias, o, m, l, sm_scale, summary=False) -> _lib.RaFwdStepParams:
     B, H, Lq, D = q.shape
     p = _lib.RaFwdStepParams()
     p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
@@ -172,7 +174,7 @@ def _fwd_params(q, k, v, bias, o, m, l, sm_scale) -> _lib.RaFwdStepParams:
             if t_.dtype != torch.float32 or not t_.is_contiguous():
                 raise ValueError("o, m, l carries must be contiguous float32 tensors")
         p.o, p.m, p.l = o.data_ptr(), m.data_ptr(), l.data_ptr()
-    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
+    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]), summary=summary)
     return p
 
 
@@ -238,7 +240,7 @@ def precompute_delta(out, do, delta=None):
     return delta
 
 
-def _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale) -> _lib.RaBwdStepParams:
+def _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, summary=False) -> _lib.RaBwdStepParams:
     B, H, Lq, D = q.shape
     p = _lib.RaBwdStepParams()
     p.B, p.H, p.Lq, p.Lk, p.D = B, H, Lq, k.shape[2], D
@@ -247,13 +249,13 @@ def _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale) -> _lib.RaB
     p.lse, p.delta = lse.data_ptr(), delta.data_ptr()
     if dq is not None:  # None: the caller fills the accumulator pointers in later, or has none
         p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
-    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]))
+    p.bias = _bias_struct(bias, q.device, (B, H, Lq, k.shape[2]), summary=summary)
     return p
 
 
 def _bwd_step(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, parts=3):
     lib = _lib.load()
-    p = _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale)
+    p = _bwd_params(q, k, v, do, lse, delta, dq, dk, dv, bias, sm_scale, summary=True)
     _lib.check("ra_bwd_step", lib.ra_bwd_step_parts(C.byref(p), parts, _stream()))
 
 

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol(lib):
 def test_struct_layout_matches_header():
     # sizes implied by the header with natural alignment on x86-64
     assert C.sizeof(_lib.RaTensor) == 32
-    assert C.sizeof(_lib.RaBias) == 8 + 16 + 16 + 16 + 16 + 16 + 8 + 8 + 24
+    assert C.sizeof(_lib.RaBias) == 8 + 16 + 16 + 16 + 16 + 16 + 8 + 8 + 24 + 8
     assert C.sizeof(_lib.RaFwdStepParams) == 24 + 3 * 32 + 24 + C.sizeof(_lib.RaBias)
     assert C.sizeof(_lib.RaBwdStepParams) == 24 + 4 * 32 + 40 + C.sizeof(_lib.RaBias)
 
@@ -130,6 +130,37 @@ def test_row_stride_limits(lib):
         p = _good_fwd()
         p.v.stride_l = good
         assert lib.ra_fwd_step_check(C.byref(p)) == 0, good
+
+
+def test_dense_map_arguments_are_checked_without_a_gpu(lib):
+    """ra_dense_map_bytes is plain arithmetic; ra_dense_map and a step that carries a summary
+    refuse bad arguments before anything is launched."""
+    assert lib.ra_dense_map_bytes(0, 0, 2, 3, 64, 64) == 4
+    assert lib.ra_dense_map_bytes(1 << 20, 0, 2, 3, 100, 250) == 2 * 4 * 8
+    assert lib.ra_dense_map_bytes(1 << 20, 1 << 16, 2, 3, 33, 1031) == 2 * 3 * 2 * 33
+    assert lib.ra_dense_map_bytes(0, 0, 0, 3, 64, 64) == 0
+    good = dict(dense_bias=0x1000, stride_b=0, stride_h=0, stride_q=64, B=1, H=1, Lq=64, Lk=64, map=0x2000)
+
+    def call(**kw):
+        a = {**good, **kw}
+        return lib.ra_dense_map(a["dense_bias"], a["stride_b"], a["stride_h"], a["stride_q"], a["B"], a["H"],
+                                a["Lq"], a["Lk"], a["map"], None)
+
+    assert call(dense_bias=None) == -1 and call(map=None) == -1          # RA_ERR_NULL
+    assert call(Lq=0) == -2 and call(B=-1) == -2                          # RA_ERR_SHAPE
+    assert call(Lk=_lib.RA_MAX_SEGMENT_SHARD + 1, stride_q=1 << 20) == -2
+    assert call(dense_bias=0x1002) == -4                                  # RA_ERR_ALIGN
+    assert call(stride_q=63) == -5 and call(stride_b=-8) == -5            # RA_ERR_BIAS
+    # a step whose dense block comes with a summary: shards of at most RA_MAX_SEGMENT_SHARD tokens
+    p = _good_fwd()
+    p.bias.flags = _lib.RA_BIAS_DENSE
+    p.bias.dense_bias, p.bias.dense_stride_q, p.bias.dense_map = 0x3000, 64, 0x4000
+    assert lib.ra_fwd_step_check(C.byref(p)) == 0
+    p.Lk = _lib.RA_MAX_SEGMENT_SHARD + 64
+    p.bias.dense_stride_q = p.Lk
+    assert lib.ra_fwd_step_check(C.byref(p)) == -2 and b"summary" in lib.ra_last_error()
+    p.bias.dense_map = None
+    assert lib.ra_fwd_step_check(C.byref(p)) == 0
 
 
 def test_bwd_step_rejects_bad_params_without_a_gpu(lib):
