@@ -44,7 +44,9 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
   // used before a shard's loops, the stash inside them, a barrier separates two shards) and
   // from a ramp table without its all-zero half.
   constexpr bool PARK2 = GENERAL;
-  constexpr bool DEFER = GENERAL;  // see the end of `iteration`
+  // generic iterations issue their tile requests last (see the end of `iteration`): all variants
+  // but the single-shard causal one
+  constexpr bool DEFER = GENERAL || MULTI;
   __shared__ unsigned char s_flag_own[(GENERAL && !PARK2) ? kMaxListTiles : 1];
   __shared__ int s_red[28];
   __shared__ int s_st[GENERAL ? 8 : 1][12];  // per wave and stretch: first iteration, end, tile_base
@@ -503,10 +505,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     // the fragments that the per-tile-term variants park in LDS are fetched from there here too:
     // they occupy no register outside the prologue
     bf16x8 qp0 = qf[0], qp1 = qf[1], qp2 = qf[2];
-    if constexpr (GENERAL) {
-      qp0 = s_q0[tid];
-      qp1 = s_q1[tid];
-    }
+    if constexpr (TIGHT) qp0 = s_q0[tid];
+    if constexpr (GENERAL) qp1 = s_q1[tid];
     if constexpr (PARK2) qp2 = s_q2[tid];
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -661,12 +661,12 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
     // this wave's share of K_{k+1}, V_k is in LDS once only the requests of barrier k-1 (K_{k+2},
     // V_{k+1}, NLD load instructions each, where they exist) are in flight
     const int pending = (k + 2 < n ? NLD : 0) + (k + 1 < n ? NLD : 0);
-    // The per-tile-term variants fetch ids with ordinary loads, which the compiler awaits without
-    // knowing of the tile loads around them: they wait for everything - except the early waves of
-    // the variants whose generic iterations issue their requests last (DEFER): there the ids are
-    // stored before the requests go out, so at this point only tile loads are in flight and the
-    // most recent ones are, as in the plain case, those of K_{k+2} and V_{k+1}.
-    const bool counted = !GENERAL || (DEFER && !late_half);
+    // The variants whose generic iterations issue their requests last (DEFER): an early wave
+    // has, as in the plain case, those of K_{k+2} and V_{k+1} as its most recent loads (the ids of
+    // the per-tile-term variants, ordinary loads, are stored before the requests go out); a late
+    // wave meets this barrier in the middle of an iteration, before its requests, so its most
+    // recent loads are a tile older than the count assumes: it waits for everything.
+    const bool counted = !DEFER || !late_half;
     if (!counted || k == 0 || pending == 0) __builtin_amdgcn_s_waitcnt(0x0f70);
     else if (pending == NLD) __builtin_amdgcn_s_waitcnt(0x0f70 | NLD);
     else __builtin_amdgcn_s_waitcnt(0x0f70 | (2 * NLD));
@@ -720,10 +720,8 @@ __global__ __launch_bounds__(kFwdThreads) void fwd_step_kernel(
 #pragma unroll
         for (int op = 0; op < PF; ++op) fr[op] = s_op_frag(kt, op);
         bf16x8 qp0 = qf[0], qp1 = qf[1], qp2 = qf[2];  // from LDS where they are parked there
-        if constexpr (GENERAL) {
-          qp0 = s_q0[tid];
-          qp1 = s_q1[tid];
-        }
+        if constexpr (TIGHT) qp0 = s_q0[tid];
+        if constexpr (GENERAL) qp1 = s_q1[tid];
         if constexpr (PARK2) qp2 = s_q2[tid];
         __builtin_amdgcn_sched_barrier(0);
         constexpr int EPO = 32 / (2 * KS);  // score elements converted per MFMA
